@@ -1,0 +1,174 @@
+/*
+ * paroatten.h - C ABI of libparoatten_hip.so: the PAROAttention hot path for AMD MI355X (gfx950).
+ *
+ * Plain pointers and sizes only.  Every pointer argument is a DEVICE pointer unless it says
+ * "host".  `stream` is a hipStream_t passed as void* (NULL = the null stream).  All strides
+ * are in ELEMENTS of the tensor they belong to.  Functions are re-entrant, keep no state
+ * between calls, never synchronise the device and never allocate; work buffers are passed in.
+ * Return value: PARO_OK or a negative PARO_ERR_* code; paro_last_error() gives the message
+ * of the last failure on the calling thread.
+ *
+ * Each entry point names the interface of the reference (jamescsq47/PAROAtten) it stands in
+ * for, as file:line relative to the reference tree.
+ */
+#ifndef PAROATTEN_H
+#define PAROATTEN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PARO_OK 0
+#define PARO_ERR_INVALID_VALUE (-1) /* bad layout / head_dim / flag: the reference throws std::invalid_argument (ValueError) */
+#define PARO_ERR_RUNTIME (-2)       /* shape / dtype / contiguity check: the reference's TORCH_CHECK (RuntimeError)        */
+#define PARO_ERR_UNSUPPORTED (-3)   /* a variant of the reference that this library does not implement                      */
+#define PARO_ERR_HIP (-4)           /* a HIP runtime call failed                                                            */
+
+#define PARO_DTYPE_F16 0
+#define PARO_DTYPE_BF16 1
+
+/* Version of this ABI (bumped when a signature changes). */
+int paro_abi_version(void);
+/* Message of the last error on this thread ("" if none). Host pointer, valid until the next call. */
+const char* paro_last_error(void);
+/* Architecture the device code was built for ("gfx950"). */
+const char* paro_build_arch(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * (1) Per-group symmetric INT8 quantisation of Q or K.
+ * Stands in for QuantInt8Kernel and its four hosts: quant_per_block_int8_cuda (6- and 5-argument
+ * overloads), quant_per_block_int8_fuse_sub_mean_cuda and quant_per_warp_int8_cuda
+ * (csrc/fused/fused.cu:64-198, 429-510, 512-592, 594-682, 685-768; csrc/fused/fused.h:19-57).
+ *
+ * x [B,H,N,D] in 16-bit `dtype`, addressed by (stride_b, stride_h, stride_n), last dim contiguous.
+ * For every group g of `group` consecutive tokens (g < n_groups, tokens >= N read as 0):
+ *   v = float(x) - float(mean[b,h,:]) (if mean != NULL) ; v *= sm_scale (if has_sm_scale)
+ *   amax = max(1e-7f, max|v|); scale[b,h,g] = amax / 127.f; out = sat_s8(rint(v * (127.f / amax)))
+ * IEEE fp32 arithmetic, round-half-even.  D in {64,128}; group in {16,32,64,128}.
+ * mean [B,H,D] in `dtype` (strides mean_stride_b/h); scale fp32 (strides scale_stride_b/h).
+ * ------------------------------------------------------------------------------------------- */
+int paro_quant_int8(const void* x, int dtype, const void* mean, int8_t* out, float* scale,
+                    int B, int H, int N, int D,
+                    int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_n,
+                    int64_t mean_stride_b, int64_t mean_stride_h,
+                    int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n,
+                    int64_t scale_stride_b, int64_t scale_stride_h,
+                    int group, int n_groups, int has_sm_scale, float sm_scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (2a) V -> FP8 (e4m3fn) with per-(b,h,channel) mean smoothing and scale, written in the
+ * MFMA-fragment tile order the attention kernel reads.
+ * Stands in for transpose_pad_permute_cuda + mean_scale_fuse_quant_cuda / scale_fuse_quant_cuda
+ * (csrc/fused/fused.cu:262-313, 316-427, 850-1083; paroattention/quant.py:224-293).  The
+ * reference's within-16 token shuffle is an NVIDIA mma fragment order; this library uses its own.
+ *
+ * v [B,Hkv,N,D] 16-bit.  v_mean, v_scale: fp32 [B,Hkv,D] (contiguous).  v8: paro_v_fp8_bytes().
+ *   mean = sum_n v / N (0 if !smooth) ; scale = max|v - mean| / 448 ; v8 = e4m3_rne((v-mean)/scale)
+ * Tile order: v8[((b*Hkv+h)*nb + kb)*64*D + ((dt*2 + mt)*64 + lane)*16 + r] holds token
+ * kb*64 + 32*mt + 8*(r/4) + 4*(lane/32) + r%4, channel 32*dt + lane%32 (tokens >= N are 0).
+ * partial: fp32 work buffer of paro_v_fp8_partial_floats() floats.
+ * ------------------------------------------------------------------------------------------- */
+int64_t paro_v_fp8_bytes(int B, int Hkv, int N, int D);
+int64_t paro_v_fp8_partial_floats(int B, int Hkv, int N, int D);
+int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_scale, float* v_mean, float* partial,
+                    int B, int Hkv, int N, int D,
+                    int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                    int smooth, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (2b) Block-sparse attention: INT8 Q.K^T on i8 MFMA (exact int32), online base-2 softmax,
+ * FP8 P.V on fp8 MFMA with fp32 accumulation, k-blocks skipped per (head, 64-row q-block).
+ * Stands in for qk_int_sv_f16_attn_kernel and the body of its host qk_int8_sv_f16_accum_f16_attn
+ * (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:44-726, 905-1080), instantiated as the reference does:
+ * 64-row q-blocks, 64-row k-blocks, q scales per 32 rows (:1022-1048).
+ *
+ * q8 [B,H,Nq,D], k8 [B,Hkv,Nk,D] int8 with element strides; q_scale fp32 [B,H,ceil(Nq/64)*2];
+ * k_scale fp32 [B,Hkv,ceil(Nk/64)]; v8/v_scale/v_mean from paro_v_fp8_pack (v_mean may be NULL).
+ * sparse: bool bytes [B,H,nbq,nbk] contiguous, nonzero = compute; if sparse_batch_stride == 0 the
+ * same [H,nbq,nbk] mask serves every batch entry.  A kept block joins the softmax support, a
+ * skipped one is as if masked with -inf; a row with no kept block outputs 0 (lse = -inf).
+ * out [B,H,Nq,D] in `out_dtype`; lse (may be NULL) fp32 [B,H,Nq], base 2: log2 sum_j 2^(s_ij*log2e).
+ * s_dump (may be NULL): int32 [B,H,nbq*64,nbk*64]; the raw Q.K^T accumulators of every computed
+ * block are stored there (debug / parity of the integer stage; untouched where skipped).
+ * D in {64,128}; is_causal in {0,1} (needs Nq == Nk).
+ * ------------------------------------------------------------------------------------------- */
+int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
+                         const float* q_scale, const float* k_scale,
+                         const float* v_scale, const float* v_mean,
+                         const uint8_t* sparse, int64_t sparse_batch_stride,
+                         void* out, int out_dtype, float* lse, int32_t* s_dump,
+                         int B, int H, int Hkv, int Nq, int Nk, int D,
+                         int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                         int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                         int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
+                         float sm_scale, int is_causal, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (2c) The reference's extension entry point in one call: V (fp16/bf16) -> FP8 tiles, then (2b).
+ * Stands in for qk_int8_sv_f16_accum_f16_attn as bound at csrc/qattn/pybind_sm80.cpp:23 /
+ * csrc/qattn/attn_cuda_sm80.h:19-31: same tensors, same integer flags (tensor_layout 0 = NHD,
+ * 1 = HND; qk_quant_gran 2 = per_warp, 3 = per_thread -> PARO_ERR_UNSUPPORTED), same checks.
+ * workspace: paro_attn_workspace_bytes() bytes of device memory (256-byte aligned).
+ * ------------------------------------------------------------------------------------------- */
+int64_t paro_attn_workspace_bytes(int B, int Hkv, int Nk, int D);
+int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, const void* v, int v_dtype,
+                             void* out, int out_dtype,
+                             const float* q_scale, const float* k_scale,
+                             const uint8_t* sparse, int64_t sparse_batch_stride,
+                             float* lse, void* workspace, int64_t workspace_bytes,
+                             int B, int H, int Hkv, int Nq, int Nk, int D,
+                             int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                             int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                             int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                             int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
+                             int tensor_layout, int is_causal, int qk_quant_gran,
+                             float sm_scale, int smooth_v, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (3) Fused 3-D RoPE + per-head F/H/W token permutation, and the inverse permutation.
+ * Stands in for the Python head loops permute_qk / permute_attn_out
+ * (paroattention/cogvideox.py:22-62, 64-110; paroattention/wan.py:25-63, 65-111), the RoPE that
+ * precedes them (cogvideox.py:167-172; wan.py:161-167) and the prototype rope_permutation
+ * (csrc/rope/rope.cu:14-48, csrc/rope/rope.cuh:9-96).
+ *
+ * Tokens [0,n_text) are text: copied through.  Image token t = (f*Hh + h)*W + w of head `head`
+ * moves to n_text + (c[p0]*S[p1] + c[p1])*S[p2] + c[p2], p = the order `orders[head]` in 0..5
+ * (0 FHW, 1 FWH, 2 HWF, 3 HFW, 4 WHF, 5 WFH), S = (F,Hh,W), c = (f,h,w).
+ * paro_rope_permute_fwd: for each of q, k (rotated if cos != NULL) and v (never rotated; any of
+ * the three may be NULL): out[b,head,new] = rot(in[b,head,old]).  Rotation of channel pairs:
+ *   o[2i] = x[2i]*cos[t,2i] - x[2i+1]*sin[t,2i] ; o[2i+1] = x[2i+1]*cos[t,2i+1] + x[2i]*sin[t,2i+1]
+ * each product and the sum rounded to fp32 (no fused multiply-add), then to `dtype`.
+ * cos, sin: fp32 [F*Hh*W, D].  orders: int32 [H] on the device.  in/out [B,H,N,D] 16-bit, must
+ * not overlap.  paro_permute_inv: out[b,head,old] = in[b,head,new] (text copied through).
+ * ------------------------------------------------------------------------------------------- */
+int paro_rope_permute_fwd(const void* q_in, const void* k_in, const void* v_in,
+                          void* q_out, void* k_out, void* v_out, int dtype,
+                          const float* cos, const float* sin, const int32_t* orders,
+                          int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                          int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_n,
+                          int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n,
+                          void* stream);
+int paro_permute_inv(const void* in, void* out, int dtype, const int32_t* orders,
+                     int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                     int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_n,
+                     int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n,
+                     void* stream);
+/* new_of_old index map of every head: idx int32 [H, F*Hh*W] (parity of the integer index law). */
+int paro_permute_index_map(int32_t* idx, const int32_t* orders, int H, int F, int Hh, int W, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * V helpers kept for API completeness of paroattention._fused (csrc/fused/fused.cu:200-260,
+ * 770-848): out_f16[b,h,n,:] = fp16(v - mean[b,h,:]) (bf16 input: subtract in bf16 first).
+ * ------------------------------------------------------------------------------------------- */
+int paro_sub_mean(const void* v, int dtype, const void* mean, void* out_f16,
+                  int B, int H, int N, int D,
+                  int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                  int64_t mean_stride_b, int64_t mean_stride_h,
+                  int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PAROATTEN_H */

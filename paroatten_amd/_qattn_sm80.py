@@ -1,0 +1,131 @@
+"""Mirror of the reference's `paroattention._qattn_sm80` extension module
+(csrc/qattn/pybind_sm80.cpp:21-27, csrc/qattn/attn_cuda_sm80.h:19-69).
+
+`qk_int8_sv_f16_accum_f16_attn` keeps the reference's positional signature, integer flags,
+validation order and messages (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:905-1080) and runs the
+gfx950 kernels of libparoatten_hip.so: V -> FP8 tiles, then INT8 QK^T / online softmax / FP8 P.V
+with fp32 accumulation.  The module keeps the reference's name although nothing here is sm80:
+callers import it under that name (paroattention/core.py:3, paroattention/cogvideox.py:13).
+
+Differences, all relaxations or added checks:
+  * `value` may be float16 (as in the reference) or bfloat16 (saves the caller's `.to(float16)`);
+  * `sparse` IS validated (the reference reads it through a raw pointer unchecked): bool or uint8,
+    on the GPU, contiguous, shape [B,H,nbq,nbk] or [H,nbq,nbk] (shared by the batch);
+  * the INT4 and INT8-P.V variants registered by the reference are experimental prototypes with
+    no working caller; they raise NotImplementedError here.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import check, load, ptr, stream_of
+
+
+def _chk(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def workspace_bytes(B, Hkv, Nk, D):
+    return int(load().paro_attn_workspace_bytes(B, Hkv, Nk, D))
+
+
+def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_scale, tensor_layout, is_causal,
+                                  qk_quant_gran, sm_scale, return_lse, sparse, *, smooth_v=True, workspace=None):
+    for t, n in ((query, "query"), (key, "key"), (value, "value"), (output, "output"),
+                 (query_scale, "query_scale"), (key_scale, "key_scale")):
+        _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
+    _chk(query.is_contiguous(), "Tensor query must be contiguous")
+    _chk(key.is_contiguous(), "Tensor key must be contiguous")
+    _chk(value.stride(-1) == 1, "Tensor value must be contiguous at the last dimension")
+    _chk(output.stride(-1) == 1, "Tensor output must be contiguous at the last dimension")
+    _chk(query_scale.is_contiguous(), "Tensor query_scale must be contiguous")
+    _chk(key_scale.is_contiguous(), "Tensor key_scale must be contiguous")
+    _chk(query.dtype == torch.int8, "Tensor query must have dtype (torch::kInt8)")
+    _chk(key.dtype == torch.int8, "Tensor key must have dtype (torch::kInt8)")
+    _chk(value.dtype in (torch.float16, torch.bfloat16), "Tensor value must have dtype (torch::kHalf)")
+    _chk(query_scale.dtype == torch.float32, "Tensor query_scale must have dtype (torch::kFloat32)")
+    _chk(key_scale.dtype == torch.float32, "Tensor key_scale must have dtype (torch::kFloat32)")
+    for t, n, d in ((query, "query", 4), (key, "key", 4), (value, "value", 4), (output, "output", 4),
+                    (query_scale, "query_scale", 3), (key_scale, "key_scale", 3)):
+        _chk(t.dim() == d, f"Tensor {n} must have dimension number ({d})")
+    D, B = query.size(3), query.size(0)
+    if tensor_layout == 0:
+        Nq, Nk, H, Hkv = query.size(1), key.size(1), query.size(2), key.size(2)
+        _chk(tuple(key.shape) == (B, Nk, Hkv, D), "Tensor key must have shape (batch_size, kv_len, num_kv_heads, head_dim)")
+        _chk(tuple(value.shape) == (B, Nk, Hkv, D), "Tensor value must have shape (batch_size, kv_len, num_kv_heads, head_dim)")
+        sn, sh = 1, 2
+    elif tensor_layout == 1:
+        Nq, Nk, H, Hkv = query.size(2), key.size(2), query.size(1), key.size(1)
+        _chk(tuple(key.shape) == (B, Hkv, Nk, D), "Tensor key must have shape (batch_size, num_kv_heads, kv_len, head_dim)")
+        _chk(tuple(value.shape) == (B, Hkv, Nk, D), "Tensor value must have shape (batch_size, num_kv_heads, kv_len, head_dim)")
+        sn, sh = 2, 1
+    else:
+        raise ValueError("tensor_layout must be 0 or 1")
+    if H % Hkv != 0:
+        raise ValueError(f"num_qo_heads ({H}) must be divisible by num_kv_heads ({Hkv})")
+    if D not in (64, 128):
+        raise ValueError(f"Unsupported head dim: {D}")
+    if is_causal not in (0, 1):
+        raise ValueError(f"Unsupported causal mode: {int(is_causal)}")
+    if qk_quant_gran not in (2, 3):
+        raise ValueError(f"Unsupported qk_quant_gran: {int(qk_quant_gran)}")
+    if return_lse not in (0, 1):
+        raise ValueError(f"Unsupported causal mode: {int(return_lse)}")  # sic: the reference's text
+    if output.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError(f"qk_int8_sv_f16_accum_f16_attn failed to dispatch data type {output.dtype}")
+    _chk(tuple(output.shape) == tuple(query.shape), "Tensor output must have the shape of query")
+    nbq, nbk = (Nq + 63) // 64, (Nk + 63) // 64
+    if qk_quant_gran == 2:
+        _chk(tuple(query_scale.shape) == (B, H, nbq * 2),
+             "Tensor query_scale must have shape (batch_size, num_qo_heads, div_ceil(qo_len, CTA_Q) * (CTA_Q / WARP_Q))")
+        _chk(tuple(key_scale.shape) == (B, Hkv, nbk),
+             "Tensor key_scale must have shape (batch_size, num_kv_heads, div_ceil(kv_len, CTA_K) * (CTA_K / WARP_K))")
+    # the mask: checked here, unlike the reference
+    _chk(sparse.is_cuda, "Tensor sparse must be on CUDA")
+    _chk(sparse.dtype in (torch.bool, torch.uint8), "Tensor sparse must have dtype (torch::kBool)")
+    _chk(sparse.is_contiguous(), "Tensor sparse must be contiguous")
+    if sparse.dim() == 4:
+        _chk(tuple(sparse.shape) == (B, H, nbq, nbk),
+             f"Tensor sparse must have shape (batch_size, num_qo_heads, {nbq}, {nbk}), got {tuple(sparse.shape)}")
+        sparse_bs = sparse.stride(0)
+    else:
+        _chk(sparse.dim() == 3 and tuple(sparse.shape) == (H, nbq, nbk),
+             f"Tensor sparse must have shape ([batch_size,] num_qo_heads, {nbq}, {nbk}), got {tuple(sparse.shape)}")
+        sparse_bs = 0
+    lse = torch.empty(0)
+    if return_lse:
+        lse = torch.empty((B, H, Nq), dtype=torch.float32, device=query.device)
+    need = workspace_bytes(B, Hkv, Nk, D)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=query.device)
+    else:
+        _chk(workspace.is_cuda and workspace.is_contiguous() and workspace.numel() * workspace.element_size() >= need,
+             f"workspace must be a contiguous GPU buffer of at least {need} bytes")
+    check(load().paro_qk_int8_sv_f16_attn(
+        ptr(query), ptr(key), ptr(value), _lib.DTYPE_CODE[value.dtype], ptr(output), _lib.DTYPE_CODE[output.dtype],
+        ptr(query_scale), ptr(key_scale), ptr(sparse), sparse_bs, ptr(lse) if return_lse else None,
+        ptr(workspace), workspace.numel() * workspace.element_size(),
+        B, H, Hkv, Nq, Nk, D,
+        query.stride(0), query.stride(sh), query.stride(sn),
+        key.stride(0), key.stride(sh), key.stride(sn),
+        value.stride(0), value.stride(sh), value.stride(sn),
+        output.stride(0), output.stride(sh), output.stride(sn),
+        tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0, stream_of(query)))
+    return lse
+
+
+def _prototype(name):
+    def fn(*args, **kwargs):
+        raise NotImplementedError(
+            f"{name}: experimental variant of the reference (INT4 Q/K or INT8 P.V) without a working "
+            "caller; gfx950 has no int4 MFMA and the INT8 P.V prototype is numerically unsound. "
+            "Use qk_int8_sv_f16_accum_f16_attn.")
+    fn.__name__ = name
+    return fn
+
+
+qk_int4_sv_f16_accum_f16_attn = _prototype("qk_int4_sv_f16_accum_f16_attn")
+qk_int4_sv_int8_accum_f16_attn = _prototype("qk_int4_sv_int8_accum_f16_attn")
+qk_int8_sv_int8_accum_f16_attn = _prototype("qk_int8_sv_int8_accum_f16_attn")

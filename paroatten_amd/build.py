@@ -1,0 +1,75 @@
+"""Build libparoatten_hip.so (device code for gfx950 only) with hipcc, in-tree.
+
+    python -m paroatten_amd.build [--force]
+
+No hipify, no torch headers: the library is plain HIP behind a C ABI (include/paroatten.h).
+IEEE fp32 arithmetic is part of the quantisation / RoPE specification, so fast-math stays off and
+fp contraction is disabled; packed-FP32 instruction selection is disabled for every source.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+LIBDIR = PKG / "lib"
+LIB = LIBDIR / "libparoatten_hip.so"
+SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "rope_permute.hip", "attn_sparse.hip"]
+ARCH = "gfx950"
+
+FLAGS = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffp-contract=off",
+    "-fno-fast-math",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def _compile(src: str, verbose: bool) -> Path:
+    obj = LIBDIR / (Path(src).stem + ".o")
+    cmd = [hipcc(), *FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{r.stdout}\n{r.stderr}")
+    if verbose and r.stderr.strip():
+        # the host pass warns that it does not know the packed-fp32 feature: harmless
+        lines = [l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip()]
+        if lines:
+            print("\n".join(lines), file=sys.stderr)
+    return obj
+
+
+def build(force: bool = True, verbose: bool = False) -> Path:
+    """Compile every HIP source and link the shared library.  Always compiles when force."""
+    LIBDIR.mkdir(exist_ok=True)
+    if not force and LIB.exists():
+        newest = max(p.stat().st_mtime for p in list(CSRC.iterdir()) + [PKG.parent / "include" / "paroatten.h"])
+        if LIB.stat().st_mtime >= newest:
+            return LIB
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+        objs = list(ex.map(lambda s: _compile(s, verbose), SOURCES))
+    cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    return LIB
+
+
+if __name__ == "__main__":
+    path = build(force="--force" in sys.argv or True, verbose=True)
+    print(path)

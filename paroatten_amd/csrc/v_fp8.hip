@@ -1,0 +1,255 @@
+// V -> FP8 (e4m3fn) per-channel quantisation with mean smoothing, written in the fragment order
+// of the P.V MFMA (v_mfma_f32_32x32x64_f8f6f4) so that the attention kernel's K-loop copies V
+// tiles straight from HBM to LDS and reads each A operand as one contiguous 16-byte piece per lane.
+//
+// Three launches, all HBM-bound and deterministic (no float atomics):
+//   v_stats    : per 256-token chunk, per channel: sum, min, max          (reads V once)
+//   v_finalize : per (b,h,channel): mean = sum/N, scale = max(max-mean, mean-min)/448
+//   v_pack     : per 64-token tile: (v-mean)/scale -> e4m3, fragment order  (reads V once more)
+// max|v-mean| over tokens equals max(max-mean, mean-min) exactly because fp32 subtraction is
+// monotonic, so no second reduction pass is needed.
+// Arithmetic follows MeanScaleKernel of the reference (csrc/fused/fused.cu:316-427) except that the
+// mean divides by the true token count.
+#include "paro_common.hpp"
+
+namespace paro {
+
+constexpr int V_CHUNK = 256;  // tokens per stats chunk
+
+template <int DT, int D>
+__global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __restrict__ v,
+                                                      float* __restrict__ partial, int N, int n_chunks,
+                                                      int64_t vs_b, int64_t vs_h, int64_t vs_n) {
+  constexpr int LPR = D / 8;
+  constexpr int ROWS = 256 / LPR;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int col = (t % LPR) * 8;
+  const unsigned short* vb = v + b * vs_b + h * vs_h + col;
+  float s[8], mn[8], mx[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) {
+    s[j] = 0.f;
+    mn[j] = INFINITY;
+    mx[j] = -INFINITY;
+  }
+#pragma unroll 4
+  for (int r = t / LPR; r < V_CHUNK; r += ROWS) {
+    const int tok = chunk * V_CHUNK + r;
+    if (tok < N) {
+      const v4i raw = *reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const unsigned w = (unsigned)raw[j >> 1];
+        const float f = F16x<DT>::to_f32((unsigned short)((j & 1) ? (w >> 16) : (w & 0xffffu)));
+        s[j] += f;
+        mn[j] = fminf(mn[j], f);
+        mx[j] = fmaxf(mx[j], f);
+      }
+    }
+  }
+  // lanes that share a column sit LPR apart
+#pragma unroll
+  for (int o = 32; o >= LPR; o >>= 1) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      s[j] += __shfl_xor(s[j], o, 64);
+      mn[j] = fminf(mn[j], __shfl_xor(mn[j], o, 64));
+      mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], o, 64));
+    }
+  }
+  __shared__ float red[4][3][D];
+  if (lane < LPR) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      red[wave][0][col + j] = s[j];
+      red[wave][1][col + j] = mn[j];
+      red[wave][2][col + j] = mx[j];
+    }
+  }
+  __syncthreads();
+  if (t < D) {
+    const float ss = (red[0][0][t] + red[1][0][t]) + (red[2][0][t] + red[3][0][t]);
+    const float mm = fminf(fminf(red[0][1][t], red[1][1][t]), fminf(red[2][1][t], red[3][1][t]));
+    const float xx = fmaxf(fmaxf(red[0][2][t], red[1][2][t]), fmaxf(red[2][2][t], red[3][2][t]));
+    float* p = partial + (((int64_t)(b * gridDim.y + h) * n_chunks + chunk) * 3) * D;
+    p[t] = ss;
+    p[D + t] = mm;
+    p[2 * D + t] = xx;
+  }
+}
+
+template <int D>
+__global__ void v_finalize_kernel(const float* __restrict__ partial, float* __restrict__ v_scale,
+                                  float* __restrict__ v_mean, int N, int n_chunks, int smooth) {
+  const int t = threadIdx.x;
+  const int64_t bh = blockIdx.x;
+  const float* p = partial + bh * n_chunks * 3 * D;
+  float s = 0.f, mn = INFINITY, mx = -INFINITY;
+  for (int c = 0; c < n_chunks; c++) {
+    s += p[(c * 3 + 0) * D + t];
+    mn = fminf(mn, p[(c * 3 + 1) * D + t]);
+    mx = fmaxf(mx, p[(c * 3 + 2) * D + t]);
+  }
+  const float mean = smooth ? s / (float)N : 0.f;
+  const float amax = fmaxf(mx - mean, mean - mn);
+  v_scale[bh * D + t] = amax / 448.0f;
+  if (v_mean) v_mean[bh * D + t] = mean;
+}
+
+template <int DT, int D>
+__global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __restrict__ v,
+                                                     uint8_t* __restrict__ v8,
+                                                     const float* __restrict__ v_scale,
+                                                     const float* __restrict__ v_mean, int N, int nb,
+                                                     int64_t vs_b, int64_t vs_h, int64_t vs_n) {
+  constexpr int LPR = D / 8;
+  constexpr int ROWS = 256 / LPR;
+  constexpr int PITCH = D + 8;  // 16-bit elements; +16 bytes keeps rows on different banks
+  __shared__ unsigned short tile[64 * PITCH];
+  const int t = threadIdx.x;
+  const int kb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int64_t bh = (int64_t)b * gridDim.y + h;
+  const int col = (t % LPR) * 8;
+  const unsigned short* vb = v + b * vs_b + h * vs_h + col;
+#pragma unroll
+  for (int r = t / LPR; r < 64; r += ROWS) {
+    const int tok = kb * 64 + r;
+    const v4i raw = (tok < N) ? *reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n) : v4i{0, 0, 0, 0};
+    *reinterpret_cast<v4i*>(&tile[r * PITCH + col]) = raw;
+  }
+  __syncthreads();
+  uint8_t* ob = v8 + (bh * nb + kb) * (int64_t)(64 * D);
+#pragma unroll
+  for (int c = t; c < 4 * D; c += 256) {  // 16-byte output pieces of this tile
+    const int lane = c & 63, mt = (c >> 6) & 1, dt = c >> 7;
+    const int ch = 32 * dt + (lane & 31);
+    const float mean = v_mean ? v_mean[bh * D + ch] : 0.f;
+    const float sc = v_scale[bh * D + ch];
+    int w[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      float f[4];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int r = 32 * mt + 8 * g + 4 * (lane >> 5) + q;
+        const float x = F16x<DT>::to_f32(tile[r * PITCH + ch]);
+        f[q] = (kb * 64 + r < N && sc > 0.f) ? (x - mean) / sc : 0.f;
+      }
+      int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+      p = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], p, true);
+      w[g] = p;
+    }
+    *reinterpret_cast<v4i*>(ob + (int64_t)c * 16) = v4i{w[0], w[1], w[2], w[3]};
+  }
+}
+
+template <int DT, int D>
+static int run_v_fp8(const void* v, uint8_t* v8, float* v_scale, float* v_mean, float* partial, int B, int Hkv,
+                     int N, int64_t vs_b, int64_t vs_h, int64_t vs_n, int smooth, hipStream_t st) {
+  const int n_chunks = ceil_div(N, V_CHUNK), nb = ceil_div(N, 64);
+  const unsigned short* vp = (const unsigned short*)v;
+  hipLaunchKernelGGL((v_stats_kernel<DT, D>), dim3(n_chunks, Hkv, B), dim3(256), 0, st, vp, partial, N, n_chunks,
+                     vs_b, vs_h, vs_n);
+  PARO_HIP(hipGetLastError());
+  hipLaunchKernelGGL((v_finalize_kernel<D>), dim3(B * Hkv), dim3(D), 0, st, (const float*)partial, v_scale,
+                     v_mean, N, n_chunks, smooth);
+  PARO_HIP(hipGetLastError());
+  hipLaunchKernelGGL((v_pack_kernel<DT, D>), dim3(nb, Hkv, B), dim3(256), 0, st, vp, v8,
+                     (const float*)v_scale, (const float*)(smooth ? v_mean : nullptr), N, nb, vs_b, vs_h, vs_n);
+  PARO_HIP(hipGetLastError());
+  return PARO_OK;
+}
+
+// out_f16 = fp16(v - mean): SubMeanKernel of the reference (csrc/fused/fused.cu:200-260); for bf16
+// input the subtraction is rounded to bf16 before the conversion to fp16, as there.
+template <int DT, int D>
+__global__ void __launch_bounds__(256) sub_mean_kernel(const unsigned short* __restrict__ v,
+                                                       const unsigned short* __restrict__ mean,
+                                                       unsigned short* __restrict__ out, int N, int64_t vs_b,
+                                                       int64_t vs_h, int64_t vs_n, int64_t ms_b, int64_t ms_h,
+                                                       int64_t os_b, int64_t os_h, int64_t os_n) {
+  constexpr int LPR = D / 8;
+  const int t = threadIdx.x;
+  const int tok = blockIdx.x * (256 / LPR) + t / LPR;
+  if (tok >= N) return;
+  const int h = blockIdx.y, b = blockIdx.z, col = (t % LPR) * 8;
+  const v4i raw = *reinterpret_cast<const v4i*>(v + b * vs_b + h * vs_h + (int64_t)tok * vs_n + col);
+  const v4i mr = *reinterpret_cast<const v4i*>(mean + b * ms_b + h * ms_h + col);
+  v4i o;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    unsigned short r2[2];
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+      const unsigned short xv = (unsigned short)(((unsigned)raw[j] >> (16 * q)) & 0xffffu);
+      const unsigned short mv = (unsigned short)(((unsigned)mr[j] >> (16 * q)) & 0xffffu);
+      float d = F16x<DT>::to_f32(xv) - F16x<DT>::to_f32(mv);
+      if constexpr (DT == PARO_DTYPE_BF16) d = F16x<PARO_DTYPE_BF16>::to_f32(F16x<PARO_DTYPE_BF16>::from_f32(d));
+      r2[q] = F16x<PARO_DTYPE_F16>::from_f32(d);
+    }
+    o[j] = (int)((unsigned)r2[0] | ((unsigned)r2[1] << 16));
+  }
+  *reinterpret_cast<v4i*>(out + b * os_b + h * os_h + (int64_t)tok * os_n + col) = o;
+}
+
+}  // namespace paro
+
+extern "C" int64_t paro_v_fp8_bytes(int B, int Hkv, int N, int D) {
+  return (int64_t)B * Hkv * paro::ceil_div(N, 64) * 64 * D;
+}
+extern "C" int64_t paro_v_fp8_partial_floats(int B, int Hkv, int N, int D) {
+  return (int64_t)B * Hkv * paro::ceil_div(N, paro::V_CHUNK) * 3 * D;
+}
+
+extern "C" int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_scale, float* v_mean,
+                               float* partial, int B, int Hkv, int N, int D, int64_t v_stride_b,
+                               int64_t v_stride_h, int64_t v_stride_n, int smooth, void* stream) {
+  using namespace paro;
+  PARO_CHECK(v && v8 && v_scale && partial, PARO_ERR_RUNTIME, "paro_v_fp8_pack: null tensor pointer");
+  PARO_CHECK(!smooth || v_mean, PARO_ERR_RUNTIME, "paro_v_fp8_pack: smoothing needs a v_mean buffer");
+  PARO_CHECK(B > 0 && Hkv > 0 && N > 0, PARO_ERR_RUNTIME, "paro_v_fp8_pack: empty shape");
+  PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
+  PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
+             "Unsupported input dtype (expect float16 or bfloat16)");
+  PARO_CHECK(v_stride_n % 8 == 0 && v_stride_h % 8 == 0 && v_stride_b % 8 == 0 && ((uintptr_t)v % 16) == 0,
+             PARO_ERR_RUNTIME, "Tensor value must be 16-byte aligned with strides that are multiples of 8");
+  PARO_CHECK(((uintptr_t)v8 % 16) == 0, PARO_ERR_RUNTIME, "paro_v_fp8_pack: v8 must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == PARO_DTYPE_F16) {
+    if (D == 64) return run_v_fp8<PARO_DTYPE_F16, 64>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
+    return run_v_fp8<PARO_DTYPE_F16, 128>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
+  }
+  if (D == 64) return run_v_fp8<PARO_DTYPE_BF16, 64>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
+  return run_v_fp8<PARO_DTYPE_BF16, 128>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
+}
+
+extern "C" int paro_sub_mean(const void* v, int dtype, const void* mean, void* out_f16, int B, int H, int N,
+                             int D, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                             int64_t mean_stride_b, int64_t mean_stride_h, int64_t out_stride_b,
+                             int64_t out_stride_h, int64_t out_stride_n, void* stream) {
+  using namespace paro;
+  PARO_CHECK(v && mean && out_f16, PARO_ERR_RUNTIME, "paro_sub_mean: null tensor pointer");
+  PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
+  PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
+             "Unsupported input dtype (expect float16 or bfloat16)");
+  PARO_CHECK(v_stride_n % 8 == 0 && v_stride_h % 8 == 0 && v_stride_b % 8 == 0 && out_stride_n % 8 == 0 &&
+                 out_stride_h % 8 == 0 && out_stride_b % 8 == 0 && mean_stride_b % 8 == 0 && mean_stride_h % 8 == 0 &&
+                 ((uintptr_t)v % 16) == 0 && ((uintptr_t)out_f16 % 16) == 0 && ((uintptr_t)mean % 16) == 0,
+             PARO_ERR_RUNTIME, "paro_sub_mean: tensors must be 16-byte aligned with strides that are multiples of 8");
+  hipStream_t st = (hipStream_t)stream;
+  const int rows = 256 / (D / 8);
+  dim3 grid(ceil_div(N, rows), H, B), block(256);
+#define PARO_SM(DTV, DV)                                                                                      \
+  hipLaunchKernelGGL((sub_mean_kernel<DTV, DV>), grid, block, 0, st, (const unsigned short*)v,                \
+                     (const unsigned short*)mean, (unsigned short*)out_f16, N, v_stride_b, v_stride_h,        \
+                     v_stride_n, mean_stride_b, mean_stride_h, out_stride_b, out_stride_h, out_stride_n)
+  if (dtype == PARO_DTYPE_F16) {
+    if (D == 64) PARO_SM(PARO_DTYPE_F16, 64); else PARO_SM(PARO_DTYPE_F16, 128);
+  } else {
+    if (D == 64) PARO_SM(PARO_DTYPE_BF16, 64); else PARO_SM(PARO_DTYPE_BF16, 128);
+  }
+#undef PARO_SM
+  PARO_HIP(hipGetLastError());
+  return PARO_OK;
+}

@@ -1,0 +1,116 @@
+"""Fused RoPE + per-head token permutation and its inverse.
+
+Replaces the reference's Python head loops `permute_qk` / `permute_attn_out`
+(paroattention/cogvideox.py:22-110, paroattention/wan.py:25-111) and the separate RoPE pass in
+front of them (cogvideox.py:167-172, wan.py:161-167) by one launch that reads Q, K, V once and
+writes them once, and one launch for the output.  All functions take HND tensors [B,H,N,D].
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import check, load, ptr, stream_of
+
+# index -> order of the (F,H,W) axes, and the inverse orders (cogvideox.py:38-45, :85-92)
+PERMUTATIONS = ((0, 1, 2), (0, 2, 1), (1, 2, 0), (1, 0, 2), (2, 1, 0), (2, 0, 1))
+PERMUTATIONS_INV = ((0, 1, 2), (0, 2, 1), (2, 0, 1), (1, 0, 2), (2, 1, 0), (1, 2, 0))
+
+
+def head_orders(permute_plan, i_block: int, device) -> torch.Tensor:
+    """int32 [H] on `device` from a plan dict {'permute': int[L,H], ...}; values checked 0..5."""
+    o = torch.as_tensor(permute_plan["permute"][i_block])
+    if o.numel() and (int(o.min()) < 0 or int(o.max()) > 5):
+        raise ValueError("permute plan entries must be in 0..5")
+    return o.to(device=device, dtype=torch.int32).contiguous()
+
+
+def _check_hnd(t: torch.Tensor, name: str):
+    _lib.require_gpu(t, name)
+    if t.dim() != 4:
+        raise RuntimeError(f"Tensor {name} must have dimension number (4)")
+    if t.dtype not in _lib.DTYPE_CODE:
+        raise RuntimeError(f"Tensor {name} must be float16 or bfloat16")
+    if t.stride(-1) != 1:
+        raise RuntimeError(f"Tensor {name} must be contiguous at the last dimension")
+
+
+def _check_orders(orders: torch.Tensor, H: int):
+    _lib.require_gpu(orders, "orders")
+    if orders.dtype != torch.int32 or orders.dim() != 1 or orders.numel() != H or not orders.is_contiguous():
+        raise RuntimeError(f"orders must be a contiguous int32 tensor of {H} entries (one per head)")
+
+
+def rope_permute(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Optional[torch.Tensor],
+                 orders: torch.Tensor, grid: Sequence[int], n_text: int,
+                 cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None
+                 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """out[b,h,perm_h(t)] = rope(in[b,h,t]) for q and k, permutation only for v; text tokens
+    [0,n_text) are copied through.  cos/sin: fp32 [F*H*W, D] (full-width tables, every frequency
+    may be repeated over its channel pair as diffusers does); None = no rotation."""
+    ref = next(t for t in (q, k, v) if t is not None)
+    _check_hnd(ref, "input")
+    B, H, N, D = ref.shape
+    for t in (q, k, v):
+        if t is not None:
+            _check_hnd(t, "input")
+            if t.shape != ref.shape or t.stride() != ref.stride() or t.dtype != ref.dtype:
+                raise RuntimeError("q, k, v must share shape, strides and dtype")
+    _check_orders(orders, H)
+    F, Hh, W = (int(x) for x in grid)
+    if cos is not None:
+        for t, n in ((cos, "cos"), (sin, "sin")):
+            _lib.require_gpu(t, n)
+            if t.dtype != torch.float32 or tuple(t.shape) != (F * Hh * W, D) or not t.is_contiguous():
+                raise RuntimeError(f"Tensor {n} must be contiguous float32 of shape ({F * Hh * W}, {D})")
+    outs = [None if t is None else torch.empty((B, H, N, D), dtype=t.dtype, device=t.device) for t in (q, k, v)]
+    o_ref = next(o for o in outs if o is not None)
+    check(load().paro_rope_permute_fwd(
+        ptr(q), ptr(k), ptr(v), ptr(outs[0]), ptr(outs[1]), ptr(outs[2]), _lib.DTYPE_CODE[ref.dtype],
+        ptr(cos), ptr(sin), ptr(orders), B, H, N, D, int(n_text), F, Hh, W,
+        ref.stride(0), ref.stride(1), ref.stride(2), o_ref.stride(0), o_ref.stride(1), o_ref.stride(2),
+        stream_of(ref)))
+    return tuple(outs)
+
+
+def permute_inverse(o: torch.Tensor, orders: torch.Tensor, grid: Sequence[int], n_text: int) -> torch.Tensor:
+    """out[b,h,t] = o[b,h,perm_h(t)]: undoes rope_permute's token order on the attention output."""
+    _check_hnd(o, "attn_out")
+    B, H, N, D = o.shape
+    _check_orders(orders, H)
+    F, Hh, W = (int(x) for x in grid)
+    out = torch.empty((B, H, N, D), dtype=o.dtype, device=o.device)
+    check(load().paro_permute_inv(ptr(o), ptr(out), _lib.DTYPE_CODE[o.dtype], ptr(orders), B, H, N, D, int(n_text),
+                                  F, Hh, W, o.stride(0), o.stride(1), o.stride(2),
+                                  out.stride(0), out.stride(1), out.stride(2), stream_of(o)))
+    return out
+
+
+def permute_index_map(orders: torch.Tensor, grid: Sequence[int]) -> torch.Tensor:
+    """int32 [H, F*H*W]: new position of every image token, per head (the integer index law)."""
+    _check_orders(orders, orders.numel())
+    F, Hh, W = (int(x) for x in grid)
+    idx = torch.empty((orders.numel(), F * Hh * W), dtype=torch.int32, device=orders.device)
+    check(load().paro_permute_index_map(ptr(idx), ptr(orders), orders.numel(), F, Hh, W, stream_of(idx)))
+    return idx
+
+
+def permute_qk(query, key, value, permute_plan, i_block, grid=(13, 30, 45), n_text=226):
+    """Drop-in for the reference's permute_qk (cogvideox.py:22-62): permutes the image tokens of
+    query, key and value IN PLACE per head and returns them.  (F,H,W) and the text length, literals
+    in the reference, are arguments with the CogVideoX values as defaults."""
+    orders = head_orders(permute_plan, i_block, query.device)
+    qo, ko, vo = rope_permute(query, key, value, orders, grid, n_text)
+    query.copy_(qo)
+    key.copy_(ko)
+    value.copy_(vo)
+    return query, key, value
+
+
+def permute_attn_out(attn_out, permute_plan, i_block, grid=(13, 30, 45), n_text=226):
+    """Drop-in for the reference's permute_attn_out (cogvideox.py:64-110), in place."""
+    orders = head_orders(permute_plan, i_block, attn_out.device)
+    attn_out.copy_(permute_inverse(attn_out, orders, grid, n_text))
+    return attn_out
