@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the PAROAttention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+Workload: BASELINE config 2, the CogVideoX-5b self-attention shape (B=2 CFG, H=48, D=64, fp16,
+N=17776 tokens = 278 blocks of 64), seeded synthetic Q/K/V with a per-channel bias on K, per-head
+banded-plus-random 64x64 block masks.  One step = one call of the reference's extension entry point
+`qk_int8_sv_f16_accum_f16_attn` (what the reference's own bench/bench.py times) at density 0.3:
+V -> FP8 tile packing followed by the block-sparse INT8-QK / FP8-PV attention kernel, inputs already
+resident in HBM.  `value` is the reference's "effective" figure 4*B*H*D*N^2 / t (dense-equivalent,
+not scaled by density); `densities` repeats the measurement at 0.5 / 0.3 / 0.2 and `path` times the
+other kernels of the path (fused RoPE+permutation, INT8 quantisation, inverse permutation).
+
+`roofline` is for the attention kernel alone: executed MFMA work 4*64*64*D per kept block, divided
+by the kernel's mean duration between HIP events recorded on the launch stream, against the 5.0
+POP/s dense INT8/FP8 MFMA peak.  `cpu_baseline` times the CPU oracle on a bounded slice.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_TOPS = 5000.0  # dense INT8 / FP8 MFMA peak of MI355X, TOP/s
+PEAK_HBM_GBS = 8000.0
+HEADLINE_DENSITY = 0.3
+DENSITIES = (0.5, 0.3, 0.2)
+# HBM bytes per attention-kernel launch at density 0.3 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/attn_sparse_cogvideox5b_pmc.txt); None until measured
+ATTN_TRAFFIC_BYTES = None
+
+
+def event_time_ms(fn, reps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def cpu_baseline(wl, density, heads=16, threads=None):
+    """The oracle (CPU port of the reference path) on a slice: B=1, `heads` heads, full N."""
+    from oracle import paro_oracle as O
+    from paroatten_amd import synth
+
+    threads = threads or min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    N, D = wl.N, wl.D
+    q, k, v = synth.make_qkv(1, heads, N, D, wl.dtype, seed=7)
+    mask = synth.make_block_mask(heads, wl.nb, density, seed=8)[None]
+    t0 = time.perf_counter()
+    km = k.float().mean(dim=2, keepdim=True).to(k.dtype)
+    q8, qs, k8, ks = O.per_warp_int8(q, k, km=km, BLKQ=64, WARPQ=32, BLKK=64)
+    O.sparse_attention(q8, k8, v, qs, ks, mask, D ** -0.5, out_dtype=wl.dtype)
+    dt = time.perf_counter() - t0
+    ops = synth.dense_equiv_ops(1, heads, N, D)
+    return {
+        "value": ops / dt / 1e12,
+        "unit": "TOPS (dense-equivalent 4*B*H*D*N^2/t)",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"oracle quant + block-sparse attention, B=1, {heads} of {wl.B * wl.H} (batch, head) pairs, "
+                  f"N={N}, D={D}, density {density}, {dt:.1f} s; per-head work is independent, so the "
+                  f"whole workload would take about {dt * wl.B * wl.H / heads:.0f} s",
+        "seconds": dt,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--workload", default="cogvideox5b", choices=["cogvideox5b", "wan14b_480p", "wan14b_720p"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU (every kernel of the path is independent per "
+              "(batch, head); nothing here uses a second GPU). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    import paroatten_amd._lib as L
+    from paroatten_amd import _qattn_sm80 as qattn
+    from paroatten_amd import permute as PM
+    from paroatten_amd import quant as Q
+    from paroatten_amd import synth
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = L.load()
+    wl = synth.WORKLOADS[args.workload]
+    B, H, D, N, nb = wl.B, wl.H, wl.D, wl.N, wl.nb
+    sm_scale = D ** -0.5
+
+    # ---- inputs, resident in HBM ----------------------------------------------------------
+    q, k, v = synth.make_qkv_device(B, H, N, D, wl.dtype, seed=0, device=dev)
+    plan = synth.make_permute_plan(1, H, seed=1)
+    orders = PM.head_orders(plan, 0, dev)
+    from paroatten_amd.rope import rope_table_cog, rope_table_wan_real
+    if args.workload == "cogvideox5b":
+        cos, sin = rope_table_cog(D, wl.grid, device=dev)
+    else:
+        cos, sin = rope_table_wan_real(D, wl.grid, device=dev)
+    qp, kp, vp = PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin)
+    km = kp.mean(dim=2, keepdim=True)
+    q8, qs, k8, ks = Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64)
+    out = torch.empty_like(q)
+    ws = torch.empty(qattn.workspace_bytes(B, H, N, D), dtype=torch.uint8, device=dev)
+    masks = {d: synth.make_block_mask(H, nb, d, seed=3, device=dev) for d in DENSITIES}
+    dense_ops = synth.dense_equiv_ops(B, H, N, D)
+
+    def entry(mask):  # the reference's extension entry point: V fp16 in, O out
+        qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, vp, out, qs, ks, 1, 0, 2, sm_scale, 0, mask, workspace=ws)
+
+    v8, vsc, vm = Q.per_channel_fp8(vp)
+
+    def attn_only(mask):  # the attention kernel alone (for the roofline)
+        L.check(lib.paro_attn_sparse_fwd(
+            L.ptr(q8), L.ptr(k8), L.ptr(v8), L.ptr(qs), L.ptr(ks), L.ptr(vsc), L.ptr(vm), L.ptr(mask), 0,
+            L.ptr(out), L.DTYPE_CODE[out.dtype], None, None, B, H, H, N, N, D,
+            q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
+            out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, L.stream_of(out)))
+
+    # ---- the timed region: exactly K steps between synchronisations -------------------------
+    head_mask = masks[HEADLINE_DENSITY]
+    for _ in range(args.warmup):
+        entry(head_mask)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        entry(head_mask)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = dense_ops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-density detail and the roofline of the attention kernel -------------------------
+    reps = max(5, min(args.steps, 50))
+    dens = {}
+    for d in DENSITIES:
+        t_entry = event_time_ms(lambda: entry(masks[d]), reps, 2)
+        t_kern = event_time_ms(lambda: attn_only(masks[d]), reps, 2)
+        ex_ops = synth.attention_ops(masks[d], D) * B
+        dens[str(d)] = {
+            "entry_ms": round(t_entry, 4),
+            "attn_kernel_ms": round(t_kern, 4),
+            "effective_tops": round(dense_ops / (t_entry * 1e-3) / 1e12, 1),
+            "effective_tops_kernel": round(dense_ops / (t_kern * 1e-3) / 1e12, 1),
+            "executed_tops_kernel": round(ex_ops / (t_kern * 1e-3) / 1e12, 1),
+            "pct_mfma_peak_kernel": round(100 * ex_ops / (t_kern * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 2),
+            "kept_blocks": int(masks[d].sum()) * B,
+        }
+    hk = dens[str(HEADLINE_DENSITY)]
+    achieved = hk["executed_tops_kernel"]
+    roofline = {
+        "kernel": "attn_sparse_kernel<64>",
+        "bound": "mfma",
+        "achieved": achieved,
+        "peak": PEAK_MFMA_TOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_MFMA_TOPS, 4),
+        "traffic": ATTN_TRAFFIC_BYTES,
+        "ops_per_launch": hk["kept_blocks"] * 4.0 * 64 * 64 * D,
+        "avg_launch_ms": hk["attn_kernel_ms"],
+    }
+
+    # ---- the bandwidth-bound kernels of the path -------------------------------------------------
+    el = B * H * N * D
+    path = {}
+    t = event_time_ms(lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), reps, 2)
+    path["rope_permute_qkv"] = {"ms": round(t, 4), "GBps": round(3 * 2 * el * 2 / t / 1e6, 1)}
+    t = event_time_ms(lambda: PM.rope_permute(q, k, None, orders, wl.grid, wl.n_text, cos, sin), reps, 2)
+    path["rope_permute_qk"] = {"ms": round(t, 4), "GBps": round(2 * 2 * el * 2 / t / 1e6, 1)}
+    t = event_time_ms(lambda: PM.permute_inverse(out, orders, wl.grid, wl.n_text), reps, 2)
+    path["permute_inverse_o"] = {"ms": round(t, 4), "GBps": round(2 * el * 2 / t / 1e6, 1)}
+    t = event_time_ms(lambda: Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64), reps, 2)
+    path["quant_int8_qk"] = {"ms": round(t, 4), "GBps": round(2 * el * 3 / t / 1e6, 1)}
+    t = event_time_ms(lambda: Q.per_channel_fp8(vp), reps, 2)
+    path["v_fp8_pack"] = {"ms": round(t, 4), "GBps": round(el * 5 / t / 1e6, 1)}
+    for p in path.values():
+        p["frac_hbm_peak"] = round(p["GBps"] / PEAK_HBM_GBS, 3)
+
+    result = {
+        "metric": "effective attn TOPS & %MFMA peak @CogVideoX-5b shape, density 0.2/0.3/0.5",
+        "value": round(value, 2),
+        "unit": "TOPS (dense-equivalent 4*B*H*D*N^2/t)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 QK^T (int32 accumulate) + fp8 e4m3 P.V (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: B={B} H={H} D={D} N={N} ({nb} blocks of 64), {str(wl.dtype)[6:]}, "
+                        f"one step = V->FP8 pack + block-sparse attention at density {HEADLINE_DENSITY}",
+            "density": HEADLINE_DENSITY,
+        },
+        "pct_mfma_peak": hk["pct_mfma_peak_kernel"],
+        "densities": dens,
+        "path": path,
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(wl, HEADLINE_DENSITY)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

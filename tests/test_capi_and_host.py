@@ -1,0 +1,122 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares, reports its architecture, and the Python mirrors reject bad arguments with the
+reference's exception types before anything touches a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "paroatten.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(paro_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    import paroatten_amd._lib as L
+    lib = L.load()
+    names = _declared_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/paroatten.h but not exported"
+        assert n in L.SIGNATURES, f"{n} has no ctypes signature"
+    assert set(L.SIGNATURES) == set(names)
+    assert lib.paro_abi_version() == 1
+    assert lib.paro_build_arch() == b"gfx950"
+    raw = ctypes.CDLL(str(L.LIB_PATH))
+    assert raw.paro_abi_version() == 1
+
+
+def test_size_queries_need_no_gpu():
+    import paroatten_amd._lib as L
+    lib = L.load()
+    assert lib.paro_v_fp8_bytes(2, 48, 17776, 64) == 2 * 48 * 278 * 64 * 64
+    assert lib.paro_v_fp8_partial_floats(1, 1, 256, 64) == 3 * 64
+    assert lib.paro_v_fp8_partial_floats(1, 1, 257, 128) == 2 * 3 * 128
+    ws = lib.paro_attn_workspace_bytes(2, 48, 17776, 64)
+    assert ws >= lib.paro_v_fp8_bytes(2, 48, 17776, 64) and ws % 256 == 0
+
+
+def test_c_abi_argument_errors_without_gpu():
+    """argument validation happens before any launch: codes and messages come back on CPU"""
+    import paroatten_amd._lib as L
+    lib = L.load()
+    rc = lib.paro_quant_int8(None, 0, None, None, None, 1, 1, 64, 64, 0, 0, 64, 0, 0, 0, 0, 64, 0, 0, 32, 2, 0, 0.0, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"null" in lib.paro_last_error()
+    buf = ctypes.create_string_buffer(4096)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 255) & ~255)
+    rc = lib.paro_quant_int8(p, 0, None, p, p, 1, 1, 64, 96, 0, 0, 96, 0, 0, 0, 0, 96, 0, 0, 32, 2, 0, 0.0, None)
+    assert rc == L.PARO_ERR_INVALID_VALUE and lib.paro_last_error() == b"Unsupported head dim: 96"
+    with pytest.raises(ValueError, match="Unsupported head dim: 96"):
+        L.check(rc)
+    rc = lib.paro_quant_int8(p, 0, None, p, p, 1, 1, 64, 64, 0, 0, 64, 0, 0, 0, 0, 64, 0, 0, 48, 2, 0, 0.0, None)
+    assert rc == L.PARO_ERR_INVALID_VALUE
+    rc = lib.paro_quant_int8(p, 0, None, p, p, 1, 1, 64, 64, 0, 0, 64, 0, 0, 0, 0, 64, 0, 0, 32, 1, 0, 0.0, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"do not cover" in lib.paro_last_error()
+    rc = lib.paro_permute_inv(p, p, 0, p, 1, 1, 100, 64, 10, 3, 5, 7, 0, 0, 64, 0, 0, 64, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
+    rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 3, 0.125, 1, None)
+    assert rc == L.PARO_ERR_UNSUPPORTED
+    with pytest.raises(NotImplementedError):
+        L.check(rc)
+    rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 16, 1, 1, 1, 64, 64, 64,
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 2, 0.125, 1, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"workspace" in lib.paro_last_error()
+    rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 7, 0, 2, 0.125, 1, None)
+    assert rc == L.PARO_ERR_INVALID_VALUE and lib.paro_last_error() == b"tensor_layout must be 0 or 1"
+
+
+def test_python_mirrors_reject_cpu_tensors_and_bad_flags():
+    from paroatten_amd import _fused, _qattn_sm80, _rope, core, quant
+    x = torch.zeros(1, 1, 64, 64, dtype=torch.float16)
+    o = torch.zeros(1, 1, 64, 64, dtype=torch.int8)
+    s = torch.zeros(1, 1, 2)
+    with pytest.raises(RuntimeError, match="Tensor input must be on CUDA"):
+        _fused.quant_per_warp_int8_cuda(x, o, s, 64, 32, 1)
+    with pytest.raises(ValueError, match="Unsupported block_size 48"):
+        _fused.quant_per_block_int8_cuda(x, o, s, 48, 1)
+    with pytest.raises(ValueError, match="Unsupported warp_block_size 8"):
+        _fused.quant_per_warp_int8_cuda(x, o, s, 64, 8, 1)
+    with pytest.raises(ValueError, match="Unknown tensor layout"):
+        quant.per_warp_int8(x, x, tensor_layout="DNH")
+    with pytest.raises(RuntimeError, match="Tensor query must be on CUDA"):
+        _qattn_sm80.qk_int8_sv_f16_accum_f16_attn(o, o, x, x, s, s, 1, 0, 2, 0.125, 0, torch.ones(1, 1, 1, 1, dtype=torch.bool))
+    with pytest.raises(NotImplementedError):
+        _qattn_sm80.qk_int4_sv_f16_accum_f16_attn()
+    with pytest.raises(NotImplementedError):
+        _fused.transpose_pad_permute_cuda(x, x, 1)
+    with pytest.raises(AssertionError, match="must be on cuda"):
+        core.paroattn_qk_int8_pv_fp16_cuda(x, x, x, torch.ones(1, 1, 1, dtype=torch.bool))
+    with pytest.raises(RuntimeError):
+        _rope.rope_permutation(x, x, torch.zeros(128), False)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    import paroatten_amd._lib as L
+    monkeypatch.setattr(L, "_lib", None)
+    monkeypatch.setenv("PAROATTEN_LIB", str(tmp_path / "nope.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        L.load()
+    monkeypatch.delenv("PAROATTEN_LIB")
+    L.load()
+
+
+def test_mask_generator_contract():
+    from paroatten_amd import synth
+    for nb, dens in ((64, 0.5), (278, 0.3), (40, 0.2)):
+        m = synth.make_block_mask(3, nb, dens, seed=1)
+        assert m.shape == (3, nb, nb) and m.dtype == torch.bool
+        target = max(int(round(dens * nb * nb)), int(((torch.arange(nb)[:, None] - torch.arange(nb)[None]).abs() <= 2).sum()))
+        assert (m.sum(dim=(1, 2)) == target).all()
+        i = torch.arange(nb)
+        assert m[:, i, i].all() and m[:, i[:-2], i[:-2] + 2].all() and m[:, i[2:], i[2:] - 2].all()
+    assert torch.equal(synth.make_block_mask(2, 16, 0.4, seed=5), synth.make_block_mask(2, 16, 0.4, seed=5))
+    plan = synth.make_permute_plan(4, 48, seed=0)
+    assert plan["permute"].shape == (4, 48) and int(plan["permute"].min()) >= 0 and int(plan["permute"].max()) <= 5

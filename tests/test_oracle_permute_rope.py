@@ -1,0 +1,97 @@
+"""Pins the permutation index law, the reshape/permute restatements and the RoPE functions of the
+oracle against torch library routines, the reference's literal tables and mathematical identities."""
+import itertools
+
+import pytest
+import torch
+
+from oracle import paro_oracle as O
+
+
+def test_literal_tables_match_reference_source():
+    # paroattention/cogvideox.py:38-45 and :85-92, held as literals here
+    assert O.PERMUTATIONS == ((0, 1, 2), (0, 2, 1), (1, 2, 0), (1, 0, 2), (2, 1, 0), (2, 0, 1))
+    assert O.PERMUTATIONS_INV == ((0, 1, 2), (0, 2, 1), (2, 0, 1), (1, 0, 2), (2, 1, 0), (1, 2, 0))
+    # the inverse table really holds the inverse orders, and all six orders are distinct
+    for p, pinv in zip(O.PERMUTATIONS, O.PERMUTATIONS_INV):
+        assert tuple(p[i] for i in pinv) == (0, 1, 2)
+    assert set(O.PERMUTATIONS) == set(itertools.permutations(range(3)))
+
+
+@pytest.mark.parametrize("grid", [(2, 3, 5), (3, 3, 3), (13, 30, 45), (21, 30, 52)])
+def test_index_law_equals_torch_permute(grid):
+    F, H, W = grid
+    n = F * H * W
+    ar = torch.arange(n).reshape(F, H, W)
+    for oid, p in enumerate(O.PERMUTATIONS):
+        new_of_old = O.permute_index_map(grid, oid)
+        old_of_new = ar.permute(*p).reshape(-1)  # library routine: out[new] = in[old_of_new[new]]
+        assert torch.equal(new_of_old[old_of_new], torch.arange(n))
+        assert sorted(new_of_old.tolist()) == list(range(n))  # a bijection
+
+
+def test_permute_qk_gather_form_and_inverse():
+    grid, n_text, B, H, D = (3, 4, 5), 7, 2, 6, 8
+    n_img = 60
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(B, H, n_text + n_img, D, generator=g)
+    k, v = q + 1, q + 2
+    plan = {"permute": torch.tensor([[0, 1, 2, 3, 4, 5]]), "empty": torch.zeros(1, 6, dtype=torch.bool)}
+    pq, pk, pv = O.permute_qk(q, k, v, plan, 0, grid, n_text)
+    for h in range(H):
+        m = O.permute_index_map(grid, h)
+        exp = torch.empty_like(q[:, h, n_text:])
+        exp[:, m] = q[:, h, n_text:]  # out[new] = in[old]
+        assert torch.equal(pq[:, h, n_text:], exp)
+        assert torch.equal(pq[:, h, :n_text], q[:, h, :n_text])  # text tokens are fixed points
+    assert torch.equal(pk, pq + 1) and torch.equal(pv, pq + 2)
+    assert torch.equal(O.permute_attn_out(pq, plan, 0, grid, n_text), q)  # inverse o forward = id
+    assert not q.data_ptr() == pq.data_ptr() and torch.equal(k, q + 1)  # inputs untouched
+
+
+def test_rope_is_a_rotation():
+    g = torch.Generator().manual_seed(1)
+    D, grid = 64, (2, 3, 4)
+    x = torch.randn(1, 2, 24, D, generator=g, dtype=torch.float64)
+    cos, sin = O.rope_table_cog(D, grid)
+    y = O.rope_apply_cog(x, cos.double(), sin.double())
+    # norm of every channel pair is preserved; position (0,0,0) is the identity
+    assert torch.allclose(y.reshape(1, 2, 24, -1, 2).norm(dim=-1), x.reshape(1, 2, 24, -1, 2).norm(dim=-1))
+    assert torch.allclose(y[:, :, 0], x[:, :, 0])
+    # agrees with the complex form: (x0 + i x1) * exp(i theta)
+    ang = torch.atan2(sin.double(), cos.double())[:, 0::2]
+    yc = torch.view_as_real(torch.view_as_complex(x.reshape(1, 2, 24, -1, 2).contiguous()) * torch.polar(torch.ones_like(ang), ang)).flatten(-2)
+    assert torch.allclose(y, yc)
+
+
+def test_rope_wan_composition_and_split():
+    D, grid = 128, (3, 4, 5)
+    f = O.rope_table_wan(D, grid)
+    assert f.shape == (1, 1, 60, 64) and f.dtype == torch.complex128
+    assert torch.allclose(f.abs(), torch.ones(1, 1, 60, 64, dtype=torch.float64))
+    ang = torch.angle(f[0, 0]).reshape(3, 4, 5, 64)
+    # channel split 22 / 21 / 21 complex pairs (44/42/42 channels): each group depends on one axis only
+    assert torch.allclose(ang[:, 0, 0, :22], ang[:, 2, 3, :22]) and torch.allclose(ang[0, :, 0, 22:43], ang[1, :, 4, 22:43])
+    assert torch.allclose(ang[0, 0, :, 43:], ang[2, 3, :, 43:])
+    # first frequency of each group is theta^0 = 1 rad per position: R(a)R(b) = R(a+b)
+    assert torch.allclose(f[0, 0].reshape(3, 4, 5, 64)[2, 0, 0, 0], f[0, 0].reshape(3, 4, 5, 64)[1, 0, 0, 0] ** 2)
+    assert float(ang[1, 0, 0, 0]) == pytest.approx(1.0) and float(ang[0, 1, 0, 22]) == pytest.approx(1.0)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(1, 2, 60, D, generator=g).bfloat16()
+    y = O.rope_apply_wan(x, f)
+    assert y.dtype == torch.bfloat16
+    assert torch.allclose(y.float().reshape(1, 2, 60, -1, 2).norm(dim=-1), x.float().reshape(1, 2, 60, -1, 2).norm(dim=-1), rtol=2e-2, atol=1e-2)
+
+
+def test_per_channel_fp8_against_library_cast():
+    g = torch.Generator().manual_seed(3)
+    v = (torch.randn(1, 2, 100, 64, generator=g) + 0.5).half()
+    v8, sc, vm = O.per_channel_fp8(v)
+    assert v8.dtype == torch.float8_e4m3fn and sc.shape == (1, 2, 64) and vm.shape == (1, 2, 64)
+    assert torch.allclose(vm, v.float().mean(dim=2))
+    centred = v.float() - vm.unsqueeze(2)
+    assert torch.allclose(sc * 448, centred.abs().amax(dim=2))
+    deq = v8.float() * sc.unsqueeze(2)
+    rel = (deq - centred).abs() / centred.abs().clamp_min(1e-3)
+    assert float(rel.max()) <= 0.0625 + 1e-3 or float(((deq - centred).abs()).max()) < 2e-2  # 3 mantissa bits
+    assert float(v8.float().abs().max()) == 448.0
