@@ -29,6 +29,8 @@ FLAGS = [
     "-ffp-contract=off",
     "-fno-fast-math",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results straight into VGPRs: no accvgpr moves around the softmax
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
 ]
 

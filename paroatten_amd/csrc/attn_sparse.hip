@@ -49,6 +49,9 @@ struct AttnParams {
 };
 
 constexpr float P_EXP_OFFSET = 8.0f;  // P~ = 2^8 * P <= 256 < 448 = max e4m3
+constexpr int S_MAGIC_BITS = 0x4B400000;  // float 1.5 * 2^23
+constexpr float S_MAGIC_F = 12582912.0f;
+constexpr int FP8_ONES = 0x38383838;  // four e4m3 1.0
 
 template <int D>
 __device__ __forceinline__ int k_swizzle(int row, int chunk) {
@@ -57,11 +60,13 @@ __device__ __forceinline__ int k_swizzle(int row, int chunk) {
 }
 
 __device__ __forceinline__ float partner_max(float x) {
-  // value of lane ^ 32 combined with own
-  return fmaxf(x, __shfl_xor(x, 32, 64));
+  // max of own value and that of lane ^ 32: v_permlane32_swap exchanges the upper half of its
+  // first operand with the lower half of its second
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP>
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE>
 __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
   constexpr int DT_TILES = D / 32;  // 32-channel tiles of O^T
@@ -169,7 +174,13 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
   for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
     for (int i = 0; i < 16; i++) o_acc[dt][i] = 0.f;
-  float m_i = -1e30f, d_i = 0.f;
+  // every row of this 32x32 tile ends up holding the row sums of P~ (only element 0 is read)
+  v16f d_acc;
+#pragma unroll
+  for (int i = 0; i < 16; i++) d_acc[i] = 0.f;
+  const v8i ones = {FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES};
+  float m_i = -1e30f;
+  float d_exact = 0.f;  // LSE only: sum of the unrounded P~ of this lane's 32 kv-columns per block
 
   load_tile(klist[0]);
   store_tile(0);
@@ -181,12 +192,14 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
     const bool more = it + 1 < cnt;
     if (more) load_tile(__builtin_amdgcn_readfirstlane((int)klist[it + 1]));
 
-    // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns
+    // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns.  The accumulators start at the
+    // bit pattern of 1.5*2^23: the int32 result then READS as the float 12582912 + S exactly
+    // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.
     v16i acc[2];
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) acc[mt][i] = 0;
+      for (int i = 0; i < 16; i++) acc[mt][i] = S_MAGIC_BITS;
     const uint8_t* kt = lds_k + buf * TILE;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
@@ -203,7 +216,7 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
 #pragma unroll
         for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) sd[32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3)] = acc[mt][i];
+          for (int i = 0; i < 16; i++) sd[32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3)] = acc[mt][i] - S_MAGIC_BITS;
       }
     }
 
@@ -211,7 +224,7 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) s[mt][i] = (float)acc[mt][i];
+      for (int i = 0; i < 16; i++) s[mt][i] = __int_as_float(acc[mt][i]);
 
     // columns past the end of K (last block) or above the diagonal (causal) leave the softmax
     const bool edge = (kb == p.nbk - 1 && (p.Nk & 63) != 0) || (CAUSAL && kb == qb);
@@ -226,21 +239,21 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
         }
     }
 
-    float smax = s[0][0];
+    float smax = fmaxf(s[0][0], s[0][1]);
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-      for (int i = 0; i < 16; i++) smax = fmaxf(smax, s[mt][i]);
-    smax = partner_max(smax);
+      for (int i = (mt == 0 ? 2 : 0); i < 16; i += 2) smax = fmaxf(fmaxf(smax, s[mt][i]), s[mt][i + 1]);
+    smax = partner_max(smax) - S_MAGIC_F;  // exact: both are integers below 2^24
 
     const float c = qsc * ksc_base[kb];
     const float m_new = fmaxf(m_i, smax * c);
     const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
     m_i = m_new;
-    const float bias = P_EXP_OFFSET - m_new;
+    const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_new);
 
-    float rs = 0.f;
     v8i pf;
+    float rs = 0.f;
 #pragma unroll
     for (int r = 0; r < 8; r++) {
       const int mt = r >> 2, i0 = 4 * (r & 3);
@@ -248,20 +261,21 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
       const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
       const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
       const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
-      rs += (p0 + p1) + (p2 + p3);
+      if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
       int w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
       w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
       pf[r] = w;
     }
-    d_i = d_i * alpha + rs;
+    if constexpr (LSE) d_exact = d_exact * alpha + rs;
     if (__ballot(alpha != 1.0f) != 0ull) {
+      d_acc[0] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
     }
 
-    // O^T += V8^T . P~^T
+    // O^T += V8^T . P~^T ; the row sums of the ROUNDED P~ come from one more MFMA against ones
     const uint8_t* vt = lds_v + buf * TILE;
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; dt++) {
@@ -270,13 +284,14 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
       const v8i a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
       o_acc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf, o_acc[dt], 0, 0, 0, 0, 0, 0);
     }
+    d_acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
 
     if (more) store_tile(buf ^ 1);
     __syncthreads();
   }
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------
-  const float d_tot = d_i + __shfl_xor(d_i, 32, 64);
+  const float d_tot = d_acc[0];
   const float inv = 1.0f / d_tot;
   if (qrow < p.Nq) {
     const float* vsc = p.v_scale + bhk * D;
@@ -296,16 +311,20 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
             v2i{(int)((unsigned)r[0] | ((unsigned)r[1] << 16)), (int)((unsigned)r[2] | ((unsigned)r[3] << 16))};
       }
     }
-    if (p.lse && lh == 0)
-      p.lse[((int64_t)b * p.H + h) * p.Nq + qrow] = m_i + __builtin_amdgcn_logf(d_tot) - P_EXP_OFFSET;
+  }
+  if constexpr (LSE) {
+    // the log-sum-exp uses the exact fp32 row sum, not the sum of the FP8-rounded weights
+    const float d_full = d_exact + __shfl_xor(d_exact, 32, 64);
+    if (p.lse && qrow < p.Nq && lh == 0)
+      p.lse[((int64_t)b * p.H + h) * p.Nq + qrow] = m_i + __builtin_amdgcn_logf(d_full) - P_EXP_OFFSET;
   }
 }
 
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP>
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
   const int grid = ((p.total + 7) / 8) * 8;
   const size_t smem = 4 * 64 * D + (((size_t)p.nbk * 2 + 15) & ~(size_t)15);
-  auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP>;
+  auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE>;
   if (smem > 48 * 1024)
     PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(128), smem, st, p);
@@ -315,8 +334,13 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
 
 template <int D, int OUT_DT>
 static int dispatch_attn(const AttnParams& p, int is_causal, bool dump, hipStream_t st) {
-  if (is_causal) return dump ? launch_attn<D, OUT_DT, true, true>(p, st) : launch_attn<D, OUT_DT, true, false>(p, st);
-  return dump ? launch_attn<D, OUT_DT, false, true>(p, st) : launch_attn<D, OUT_DT, false, false>(p, st);
+  const bool lse = p.lse != nullptr;
+  if (dump) {  // debug path: one instantiation per causal mode, always with the exact row sum
+    if (is_causal) return launch_attn<D, OUT_DT, true, true, true>(p, st);
+    return launch_attn<D, OUT_DT, false, true, true>(p, st);
+  }
+  if (is_causal) return lse ? launch_attn<D, OUT_DT, true, false, true>(p, st) : launch_attn<D, OUT_DT, true, false, false>(p, st);
+  return lse ? launch_attn<D, OUT_DT, false, false, true>(p, st) : launch_attn<D, OUT_DT, false, false, false>(p, st);
 }
 
 }  // namespace paro
