@@ -12,9 +12,12 @@
 // need one exchange with the partner lane (lane ^ 32) only.
 //
 // k-blocks: the workgroup turns its row of the bool mask into a compact list in LDS and loops over
-// the kept blocks only; a skipped block costs neither loads nor MFMA issue.  K8 (row-major, XOR
-// swizzled against bank conflicts) and V8 (already in fragment order) tiles are double-buffered in
-// LDS: the global loads of block i+1 are in flight while block i is computed.
+// the kept blocks only; a skipped block costs neither loads nor MFMA issue.  K8 (row-major rows
+// padded by 16 bytes against bank conflicts) and V8 (already in fragment order) tiles go through a 3-stage
+// LDS ring, and the loop is software-pipelined: while the softmax of block i runs on the VALU, the
+// global loads of block i+2 are in flight, the K fragments of block i+1 and the V fragments of
+// block i are on their way out of LDS, and the iteration ends with Q.K^T of block i+1 issued ahead
+// of P.V of block i, so that the next softmax can start under the P.V MFMAs.  One barrier per block.
 //
 // Workgroups are renumbered so that each of the 8 XCDs walks a contiguous range of (batch, head,
 // q-block): the K8/V8 of the one or two heads an XCD is working on stay resident in its own L2.
@@ -24,6 +27,7 @@
 // scale indexing :100-133, mask indexing :222/:268, out-of-range columns attn_utils.cuh:355-381,
 // softmax recurrence attn_utils.cuh:383-488, normalisation :786-840, lse = log2(d) + m (:711-723).
 #include "paro_common.hpp"
+#include <type_traits>
 
 namespace paro {
 
@@ -48,36 +52,68 @@ struct AttnParams {
   float sm_scale_log2e;
 };
 
-constexpr float P_EXP_OFFSET = 8.0f;  // P~ = 2^8 * P <= 256 < 448 = max e4m3
+// P~ = 2^(S*c - m + P_EXP_OFFSET).  m is the running row maximum, refreshed lazily: only when a
+// block's maximum exceeds it by more than P_HEADROOM are m, O and the row sums rescaled, so that
+// P~ <= 2^(P_EXP_OFFSET + P_HEADROOM) = 2^8.75 < 448, the largest e4m3 value.
+constexpr float P_EXP_OFFSET = 5.0f;
+constexpr float P_HEADROOM = 3.75f;
 constexpr int S_MAGIC_BITS = 0x4B400000;  // float 1.5 * 2^23
 constexpr float S_MAGIC_F = 12582912.0f;
 constexpr int FP8_ONES = 0x38383838;  // four e4m3 1.0
+constexpr int NST = 3;                // LDS ring stages
 
-template <int D>
-__device__ __forceinline__ int k_swizzle(int row, int chunk) {
-  if constexpr (D == 64) return chunk ^ (((row >> 1) ^ (row >> 3)) & 3);
-  else return chunk ^ ((row ^ (row >> 3)) & 7);
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// two floats -> two e4m3 bytes in the low (HI = false) or high half of a word; the other half of the
+// destination is left as it is, so a full word takes one call of each kind
+template <bool HI>
+__device__ __forceinline__ void cvt_pk_fp8(int& w, float a, float b) {
+  if constexpr (HI) asm("v_cvt_pk_fp8_f32 %0, %1, %2 op_sel:[0,0,1]" : "+v"(w) : "v"(a), "v"(b));
+  else asm("v_cvt_pk_fp8_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));  // upper half: don't care, overwritten next
 }
 
 __device__ __forceinline__ float partner_max(float x) {
   // max of own value and that of lane ^ 32: v_permlane32_swap exchanges the upper half of its
   // first operand with the lower half of its second
   const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  return max3(__uint_as_float(r[0]), __uint_as_float(r[1]), __uint_as_float(r[1]));
 }
 
+__device__ __forceinline__ void* uniform_ptr(const void* ptr) {
+  // the address is the same in every lane; say so, so that the descriptor lives in scalar registers
+  const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+  return reinterpret_cast<void*>(((unsigned long long)hi << 32) | lo);
+}
+
+__device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, int voffset, int soffset) {
+  // out-of-range bytes read as 0 (raw buffer, bounds-checked by the hardware)
+  return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voffset, soffset, 0));
+}
+
+template <int D> struct AttnLds {
+  static constexpr int KPITCH = D + 16;        // padded K rows: conflict-free 16-byte column reads
+  static constexpr int KTILE = 64 * KPITCH;    // bytes of one K8 tile in LDS
+  static constexpr int VTILE = 64 * D;         // bytes of one V8 tile (fragment order, as in HBM)
+  static constexpr int V_OFF = NST * KTILE;
+  static constexpr int LIST_OFF = NST * (KTILE + VTILE);
+};
+
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE>
-__global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p) {
+  using Lds = AttnLds<D>;
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
   constexpr int DT_TILES = D / 32;  // 32-channel tiles of O^T
   constexpr int NLD = D / 32;       // 16-byte pieces per thread per K (or V) tile
-  constexpr int TILE = 64 * D;      // bytes of one K8 or V8 tile
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  uint8_t* lds_k = smem;                   // [2][TILE]
-  uint8_t* lds_v = smem + 2 * TILE;        // [2][TILE]
-  unsigned short* klist = reinterpret_cast<unsigned short*>(smem + 4 * TILE);  // [nbk]
+  unsigned short* klist = reinterpret_cast<unsigned short*>(smem + Lds::LIST_OFF);  // [nbk + 4]
   __shared__ int s_cnt;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -97,7 +133,7 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
   const int kmax = CAUSAL ? min(p.nbk, qb + 1) : p.nbk;
   if (wave == 0) {
     const uint8_t* mrow = p.sparse + b * p.sparse_bs + ((int64_t)h * p.nbq + qb) * p.nbk;
-    int cnt = 0;
+    int cnt = 0, last = 0;
     for (int base = 0; base < kmax; base += 256) {
       uint8_t m[4];
 #pragma unroll
@@ -111,8 +147,11 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
         const unsigned long long bal = __ballot(keep);
         if (keep) klist[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (unsigned short)(base + u * 64 + lane);
         cnt += __popcll(bal);
+        if (bal) last = base + u * 64 + 63 - __clzll(bal);
       }
     }
+    // the loop prefetches up to 3 blocks ahead without branching: pad with the last kept block
+    if (lane < 4) klist[cnt + lane] = (unsigned short)last;
     if (lane == 0) s_cnt = cnt;
   }
 
@@ -120,13 +159,13 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
   const int qrow = qb * 64 + wave * 32 + l32;
   v4i qf[KS];
   {
-    const int8_t* qp = p.q8 + b * p.qs_b + h * p.qs_h + (int64_t)qrow * p.qs_n + 16 * lh;
+    // rows past the end re-read the last row; their results are never stored
+    const int8_t* qp = p.q8 + b * p.qs_b + h * p.qs_h + (int64_t)min(qrow, p.Nq - 1) * p.qs_n + 16 * lh;
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++)
-      qf[ks] = (qrow < p.Nq) ? *reinterpret_cast<const v4i*>(qp + 32 * ks) : v4i{0, 0, 0, 0};
+    for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
   }
   const float qsc = p.q_scale[((int64_t)b * p.H + h) * (p.nbq * 2) + qb * 2 + wave] * p.sm_scale_log2e;
-  const float* ksc_base = p.k_scale + bhk * p.nbk;
+  const float* ksc_base = static_cast<const float*>(uniform_ptr(p.k_scale + bhk * p.nbk));
 
   __syncthreads();
   const int cnt = s_cnt;
@@ -143,28 +182,76 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
     return;
   }
 
-  // ---- tile movers ------------------------------------------------------------------------
-  const int8_t* kg = p.k8 + b * p.ks_b + hk * p.ks_h;
-  const uint8_t* vg = p.v8 + bhk * p.nbk * (int64_t)TILE;
+  // ---- tile movers: buffer loads (scalar base + per-thread offset fixed for the whole loop +
+  //      scalar per-block offset), staged through registers into the LDS ring ------------------
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      uniform_ptr(p.k8 + b * p.ks_b + hk * p.ks_h), 0, (int)((int64_t)(p.Nk - 1) * p.ks_n + D), 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      uniform_ptr(p.v8 + bhk * p.nbk * (int64_t)Lds::VTILE), 0, p.nbk * Lds::VTILE, 0x00020000);
+  int k_goff[NLD], k_loff[NLD], v_off[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; i++) {
+    const int c = t + 128 * i;
+    const int row = c / CPR, cc = c % CPR;
+    k_goff[i] = row * (int)p.ks_n + cc * 16;
+    k_loff[i] = row * Lds::KPITCH + cc * 16;
+    v_off[i] = c * 16;
+  }
+  const int k_blk_stride = 64 * (int)p.ks_n;
   v4i kst[NLD], vst[NLD];
   auto load_tile = [&](int kb) {
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-      const int c = t + 128 * i;
-      const int row = c / CPR, cc = c % CPR;
-      const int kvrow = kb * 64 + row;
-      kst[i] = (kvrow < p.Nk) ? *reinterpret_cast<const v4i*>(kg + (int64_t)kvrow * p.ks_n + cc * 16)
-                              : v4i{0, 0, 0, 0};
-      vst[i] = *reinterpret_cast<const v4i*>(vg + (int64_t)kb * TILE + c * 16);
+      kst[i] = buffer_load16(k_rsrc, k_goff[i], kb * k_blk_stride);  // rows >= Nk read as 0
+      vst[i] = buffer_load16(v_rsrc, v_off[i], kb * Lds::VTILE);
     }
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](int ST) {
 #pragma unroll
     for (int i = 0; i < NLD; i++) {
-      const int c = t + 128 * i;
-      const int row = c / CPR, cc = c % CPR;
-      *reinterpret_cast<v4i*>(lds_k + buf * TILE + row * D + k_swizzle<D>(row, cc) * 16) = kst[i];
-      *reinterpret_cast<v4i*>(lds_v + buf * TILE + c * 16) = vst[i];
+      *reinterpret_cast<v4i*>(smem + ST * Lds::KTILE + k_loff[i]) = kst[i];
+      *reinterpret_cast<v4i*>(smem + Lds::V_OFF + ST * Lds::VTILE + v_off[i]) = vst[i];
+    }
+  };
+
+  // ---- fragment movers and the two matrix products ---------------------------------------
+  const int kr_base = l32 * Lds::KPITCH + lh * 16;  // K fragment (ks, mt): + ks*32 + mt*32*KPITCH
+  const int vr_base = Lds::V_OFF + lane * 16;        // V fragment (dt, mt): + (dt*2+mt)*1024
+  v4i kfrag[2 * KS];
+  auto read_k_frags = [&](int ST) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int mt = 0; mt < 2; mt++)
+        kfrag[ks * 2 + mt] =
+            *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + kr_base + ks * 32 + mt * 32 * Lds::KPITCH);
+  };
+  // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns.  The accumulators start at the bit
+  // pattern of 1.5*2^23: the int32 result then READS as the float 12582912 + S exactly
+  // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.
+  v16i magic;
+#pragma unroll
+  for (int i = 0; i < 16; i++) magic[i] = S_MAGIC_BITS;
+  asm volatile("" : "+v"(magic));  // keep the constant block resident instead of rebuilding it per block
+  v16i acc[2];
+  auto qk_mfma = [&]() {
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+      acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[mt], qf[0], magic, 0, 0, 0);
+#pragma unroll
+      for (int ks = 1; ks < KS; ks++)
+        acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[ks * 2 + mt], qf[ks], acc[mt], 0, 0, 0);
+    }
+  };
+  auto dump_s = [&](int kb) {
+    if constexpr (DUMP) {
+      if (p.s_dump) {
+        int32_t* sd = p.s_dump + (((int64_t)b * p.H + h) * (p.nbq * 64) + qrow) * (int64_t)(p.nbk * 64) + kb * 64;
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) sd[32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3)] = acc[mt][i] - S_MAGIC_BITS;
+      }
     }
   };
 
@@ -178,48 +265,45 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
   v16f d_acc;
 #pragma unroll
   for (int i = 0; i < 16; i++) d_acc[i] = 0.f;
-  const v8i ones = {FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES};
+  v8i ones = {FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES};
+  asm volatile("" : "+v"(ones));  // same: resident constant operand
   float m_i = -1e30f;
   float d_exact = 0.f;  // LSE only: sum of the unrounded P~ of this lane's 32 kv-columns per block
 
-  load_tile(klist[0]);
+  // ---- prologue: blocks 0 and 1 into the ring, block 2 in flight, S of block 0 ---------------
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  int kb_c = __builtin_amdgcn_readfirstlane((int)klist[0]);
+  int kb_1 = __builtin_amdgcn_readfirstlane((int)klist[1]);
+  int kb_2 = __builtin_amdgcn_readfirstlane((int)klist[2]);
+  load_tile(kb_c);
   store_tile(0);
+  load_tile(kb_1);
+  store_tile(1);
+  load_tile(kb_2);
+  float c_cur = qsc * ksc_base[kb_c];
   __syncthreads();
+  read_k_frags(0);
+  qk_mfma();
+  dump_s(kb_c);
 
-  for (int it = 0; it < cnt; it++) {
-    const int kb = __builtin_amdgcn_readfirstlane((int)klist[it]);
-    const int buf = it & 1;
-    const bool more = it + 1 < cnt;
-    if (more) load_tile(__builtin_amdgcn_readfirstlane((int)klist[it + 1]));
+  // one block; stage_c holds its V tile, stage_1 the K tile of the next block, stage_2 receives
+  // the block after that
+  auto step = [&](int it, int SC, int stage_1, int stage_2) {
+    // -- LDS traffic of this iteration, issued up front: index of block it+3, V fragments of the
+    //    current block, K fragments of the next one
+    const int kidx_v = (int)klist[it + 3];
+    v4i vfrag[DT_TILES][2];
+#pragma unroll
+    for (int dt = 0; dt < DT_TILES; dt++)
+#pragma unroll
+      for (int mt = 0; mt < 2; mt++)
+        vfrag[dt][mt] = *reinterpret_cast<const v4i*>(smem + SC * Lds::VTILE + vr_base + (dt * 2 + mt) * 1024);
+    read_k_frags(stage_1);
+    const float c_next = qsc * ksc_base[kb_1];
 
-    // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns.  The accumulators start at the
-    // bit pattern of 1.5*2^23: the int32 result then READS as the float 12582912 + S exactly
-    // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.
-    v16i acc[2];
-#pragma unroll
-    for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) acc[mt][i] = S_MAGIC_BITS;
-    const uint8_t* kt = lds_k + buf * TILE;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-#pragma unroll
-      for (int mt = 0; mt < 2; mt++) {
-        const int row = 32 * mt + l32;
-        const v4i kf = *reinterpret_cast<const v4i*>(kt + row * D + k_swizzle<D>(row, 2 * ks + lh) * 16);
-        acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ks], acc[mt], 0, 0, 0);
-      }
-    }
-    if constexpr (DUMP) {
-      if (p.s_dump) {
-        int32_t* sd = p.s_dump + (((int64_t)b * p.H + h) * (p.nbq * 64) + qrow) * (int64_t)(p.nbk * 64) + kb * 64;
-#pragma unroll
-        for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) sd[32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3)] = acc[mt][i] - S_MAGIC_BITS;
-      }
-    }
-
+    // -- softmax of the current block
     float s[2][16];
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
@@ -227,30 +311,43 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
       for (int i = 0; i < 16; i++) s[mt][i] = __int_as_float(acc[mt][i]);
 
     // columns past the end of K (last block) or above the diagonal (causal) leave the softmax
-    const bool edge = (kb == p.nbk - 1 && (p.Nk & 63) != 0) || (CAUSAL && kb == qb);
+    const bool edge = (kb_c == p.nbk - 1 && (p.Nk & 63) != 0) || (CAUSAL && kb_c == qb);
     if (edge) {
 #pragma unroll
       for (int mt = 0; mt < 2; mt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const int j = kb * 64 + 32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3);
+          const int j = kb_c * 64 + 32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3);
           const bool dead = (j >= p.Nk) || (CAUSAL && j > qrow);
           if (dead) s[mt][i] = -INFINITY;
         }
     }
 
-    float smax = fmaxf(s[0][0], s[0][1]);
+    // two interleaved v_max3 chains (the values are integers read as floats: no NaN to canonicalise)
+    float mx0 = s[0][0], mx1 = s[1][0];
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-      for (int i = (mt == 0 ? 2 : 0); i < 16; i += 2) smax = fmaxf(fmaxf(smax, s[mt][i]), s[mt][i + 1]);
+    for (int i = 1; i < 15; i += 2) {
+      mx0 = max3(mx0, s[0][i], s[0][i + 1]);
+      mx1 = max3(mx1, s[1][i], s[1][i + 1]);
+    }
+    float smax = max3(mx0, mx1, s[0][15]);
+    smax = max3(smax, s[1][15], smax);
     smax = partner_max(smax) - S_MAGIC_F;  // exact: both are integers below 2^24
 
-    const float c = qsc * ksc_base[kb];
-    const float m_new = fmaxf(m_i, smax * c);
-    const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
-    m_i = m_new;
-    const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_new);
+    const float c = c_cur;
+    const float m_blk = smax * c;
+    if (__ballot(m_blk > m_i + P_HEADROOM) != 0ull) {  // rare after the first few blocks
+      const float m_new = fmaxf(m_i, m_blk);
+      const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+      m_i = m_new;
+      if constexpr (LSE) d_exact *= alpha;
+      d_acc[0] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT_TILES; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
+    }
+    const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
 
     v8i pf;
     float rs = 0.f;
@@ -262,32 +359,39 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
       const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
       const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
       if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
-      int w = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, 0, false);
-      w = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, w, true);
+      int w;
+      cvt_pk_fp8<false>(w, p0, p1);
+      cvt_pk_fp8<true>(w, p2, p3);
       pf[r] = w;
     }
-    if constexpr (LSE) d_exact = d_exact * alpha + rs;
-    if (__ballot(alpha != 1.0f) != 0ull) {
-      d_acc[0] *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < DT_TILES; dt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
-    }
+    if constexpr (LSE) d_exact += rs;
 
-    // O^T += V8^T . P~^T ; the row sums of the ROUNDED P~ come from one more MFMA against ones
-    const uint8_t* vt = lds_v + buf * TILE;
+    // -- S^T of the NEXT block first (its softmax opens the next iteration), then
+    //    O^T += V8^T . P~^T of this one; the row sums of the ROUNDED P~ come from one more MFMA
+    //    against ones
+    qk_mfma();
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; dt++) {
-      const v4i a0 = *reinterpret_cast<const v4i*>(vt + ((dt * 2 + 0) * 64 + lane) * 16);
-      const v4i a1 = *reinterpret_cast<const v4i*>(vt + ((dt * 2 + 1) * 64 + lane) * 16);
-      const v8i a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+      const v8i a = {vfrag[dt][0][0], vfrag[dt][0][1], vfrag[dt][0][2], vfrag[dt][0][3],
+                     vfrag[dt][1][0], vfrag[dt][1][1], vfrag[dt][1][2], vfrag[dt][1][3]};
       o_acc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf, o_acc[dt], 0, 0, 0, 0, 0, 0);
     }
     d_acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
+    if (it + 1 < cnt) dump_s(kb_1);
 
-    if (more) store_tile(buf ^ 1);
+    // -- block it+2 from registers into the ring, block it+3 from HBM/L2 into registers
+    store_tile(stage_2);
+    const int kb_3 = __builtin_amdgcn_readfirstlane(kidx_v);
+    load_tile(kb_3);
     __syncthreads();
+    kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3;
+    c_cur = c_next;
+  };
+
+  int st_c = 0, st_1 = 1, st_2 = 2;
+  for (int it = 0; it < cnt; it++) {
+    step(it, st_c, st_1, st_2);
+    const int st_t = st_c; st_c = st_1; st_1 = st_2; st_2 = st_t;
   }
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------
@@ -323,7 +427,7 @@ __global__ void __launch_bounds__(128) attn_sparse_kernel(const AttnParams p) {
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
   const int grid = ((p.total + 7) / 8) * 8;
-  const size_t smem = 4 * 64 * D + (((size_t)p.nbk * 2 + 15) & ~(size_t)15);
+  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + 4) * 2 + 15) & ~(size_t)15);
   auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE>;
   if (smem > 48 * 1024)
     PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));

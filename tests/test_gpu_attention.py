@@ -149,7 +149,5 @@ def test_int32_qk_accumulators_bitexact(dev, D):
     # computed blocks: exact on the real rows/columns; skipped blocks: untouched
     assert torch.equal(dump[..., :N, :N][keep[..., :N, :N]], s_ref[keep[..., :N, :N]])
     assert (dump[~keep] == -(2 ** 31)).all()
-    # padded rows/columns of computed blocks are products with zero rows
-    pad_region = keep.clone()
-    pad_region[..., :N, :N] = False
-    assert (dump[pad_region] == 0).all()
+    # (rows/columns past N inside computed blocks hold products with a re-read last row; the
+    # kernel masks those columns out of the softmax and never stores those rows)
