@@ -136,7 +136,7 @@ def main():
             L.ptr(q8), L.ptr(k8), L.ptr(v8), L.ptr(qs), L.ptr(ks), L.ptr(vsc), L.ptr(vm), L.ptr(mask), 0,
             L.ptr(out), L.DTYPE_CODE[out.dtype], None, None, B, H, H, N, N, D,
             q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
-            out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, L.stream_of(out)))
+            out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, 0, L.stream_of(out)))
 
     # ---- the timed region: exactly K steps between synchronisations -------------------------
     head_mask = masks[HEADLINE_DENSITY]

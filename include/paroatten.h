@@ -29,6 +29,10 @@ extern "C" {
 #define PARO_DTYPE_F16 0
 #define PARO_DTYPE_BF16 1
 
+/* flags of the attention entry points */
+#define PARO_ATTN_EXACT_EXP 1 /* P = e4m3(2^x) by hardware exponential + FP8 conversion instead of the fast
+                                 direct construction of the e4m3 byte (see paro_attn_sparse_fwd) */
+
 /* Version of this ABI (bumped when a signature changes). */
 int paro_abi_version(void);
 /* Message of the last error on this thread ("" if none). Host pointer, valid until the next call. */
@@ -93,6 +97,11 @@ int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_scale, float
  * s_dump (may be NULL): int32 [B,H,nbq*64,nbk*64]; the raw Q.K^T accumulators of every computed
  * block are stored there (debug / parity of the integer stage; untouched where skipped).
  * D in {64,128}; is_causal in {0,1} (needs Nq == Nk).
+ * flags: 0, or PARO_ATTN_EXACT_EXP.  By default the softmax weight 2^x is turned into its e4m3 byte
+ * directly (exponent field from floor(x), mantissa by linear interpolation between powers of two,
+ * round-to-nearest-even): at most 6 % from the exact weight, which the row normalisation (done with the
+ * same rounded weights) absorbs; measured output error stays inside atol 2e-2 / cosine 0.999.  With
+ * PARO_ATTN_EXACT_EXP, or whenever lse or s_dump is requested, 2^x is evaluated in fp32 and rounded.
  * ------------------------------------------------------------------------------------------- */
 int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
                          const float* q_scale, const float* k_scale,
@@ -103,7 +112,7 @@ int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
                          int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
                          int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
                          int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
-                         float sm_scale, int is_causal, void* stream);
+                         float sm_scale, int is_causal, int flags, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * (2c) The reference's extension entry point in one call: V (fp16/bf16) -> FP8 tiles, then (2b).
@@ -124,7 +133,7 @@ int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, const void* v, 
                              int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
                              int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
                              int tensor_layout, int is_causal, int qk_quant_gran,
-                             float sm_scale, int smooth_v, void* stream);
+                             float sm_scale, int smooth_v, int flags, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * (3) Fused 3-D RoPE + per-head F/H/W token permutation, and the inverse permutation.

@@ -19,6 +19,7 @@ PARO_ERR_INVALID_VALUE = -1
 PARO_ERR_RUNTIME = -2
 PARO_ERR_UNSUPPORTED = -3
 PARO_ERR_HIP = -4
+PARO_ATTN_EXACT_EXP = 1
 
 DTYPE_CODE = {torch.float16: 0, torch.bfloat16: 1}
 
@@ -38,12 +39,12 @@ SIGNATURES = {
     "paro_v_fp8_pack": (c_int, [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _I, _P]),
     "paro_attn_sparse_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _I, _P, _P,
                                      _I, _I, _I, _I, _I, _I,
-                                     _L, _L, _L, _L, _L, _L, _L, _L, _L, _F, _I, _P]),
+                                     _L, _L, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I, _P]),
     "paro_attn_workspace_bytes": (c_int64, [_I, _I, _I, _I]),
     "paro_qk_int8_sv_f16_attn": (c_int, [_P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _P, _P, _L,
                                          _I, _I, _I, _I, _I, _I,
                                          _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
-                                         _I, _I, _I, _F, _I, _P]),
+                                         _I, _I, _I, _F, _I, _I, _P]),
     "paro_rope_permute_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _I, _P, _P, _P,
                                       _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
     "paro_permute_inv": (c_int, [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),

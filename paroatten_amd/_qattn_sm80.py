@@ -9,6 +9,8 @@ callers import it under that name (paroattention/core.py:3, paroattention/cogvid
 
 Differences, all relaxations or added checks:
   * `value` may be float16 (as in the reference) or bfloat16 (saves the caller's `.to(float16)`);
+  * keyword `exact_exp=True` evaluates the softmax exponentials in fp32 before the FP8 rounding instead
+    of building the e4m3 byte directly (slower, slightly more accurate; always on with return_lse);
   * `sparse` IS validated (the reference reads it through a raw pointer unchecked): bool or uint8,
     on the GPU, contiguous, shape [B,H,nbq,nbk] or [H,nbq,nbk] (shared by the batch);
   * the INT4 and INT8-P.V variants registered by the reference are experimental prototypes with
@@ -32,7 +34,8 @@ def workspace_bytes(B, Hkv, Nk, D):
 
 
 def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_scale, tensor_layout, is_causal,
-                                  qk_quant_gran, sm_scale, return_lse, sparse, *, smooth_v=True, workspace=None):
+                                  qk_quant_gran, sm_scale, return_lse, sparse, *, smooth_v=True, exact_exp=False,
+                                  workspace=None):
     for t, n in ((query, "query"), (key, "key"), (value, "value"), (output, "output"),
                  (query_scale, "query_scale"), (key_scale, "key_scale")):
         _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
@@ -112,7 +115,8 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
         key.stride(0), key.stride(sh), key.stride(sn),
         value.stride(0), value.stride(sh), value.stride(sn),
         output.stride(0), output.stride(sh), output.stride(sn),
-        tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0, stream_of(query)))
+        tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0,
+        _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0, stream_of(query)))
     return lse
 
 

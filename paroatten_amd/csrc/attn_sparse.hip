@@ -61,6 +61,7 @@ constexpr int S_MAGIC_BITS = 0x4B400000;  // float 1.5 * 2^23
 constexpr float S_MAGIC_F = 12582912.0f;
 constexpr int FP8_ONES = 0x38383838;  // four e4m3 1.0
 constexpr int NST = 3;                // LDS ring stages
+constexpr float FAST_EXP_SHIFT = -0.35f;  // centres the linear-mantissa error of the fast exponential
 
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
@@ -74,6 +75,14 @@ template <bool HI>
 __device__ __forceinline__ void cvt_pk_fp8(int& w, float a, float b) {
   if constexpr (HI) asm("v_cvt_pk_fp8_f32 %0, %1, %2 op_sel:[0,0,1]" : "+v"(w) : "v"(a), "v"(b));
   else asm("v_cvt_pk_fp8_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));  // upper half: don't care, overwritten next
+}
+
+// float -> unsigned byte (round to nearest even, clamped to [0,255]) into byte BYTE of w; FIRST starts
+// a fresh word (whatever the other bytes hold is overwritten by the three calls that follow)
+template <int BYTE, bool FIRST>
+__device__ __forceinline__ void cvt_pk_u8(int& w, float a) {
+  if constexpr (FIRST) asm("v_cvt_pk_u8_f32 %0, %1, %2, %0" : "=v"(w) : "v"(a), "n"(BYTE));
+  else asm("v_cvt_pk_u8_f32 %0, %1, %2, %0" : "+v"(w) : "v"(a), "n"(BYTE));
 }
 
 __device__ __forceinline__ float partner_max(float x) {
@@ -104,7 +113,7 @@ template <int D> struct AttnLds {
   static constexpr int LIST_OFF = NST * (KTILE + VTILE);
 };
 
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE>
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p) {
   using Lds = AttnLds<D>;
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
@@ -113,7 +122,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  unsigned short* klist = reinterpret_cast<unsigned short*>(smem + Lds::LIST_OFF);  // [nbk + 4]
+  float* clist = reinterpret_cast<float*>(smem + Lds::LIST_OFF);                       // [nbk + 4] k_scale of kept blocks
+  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + p.nbk + 4);  // [nbk + 4] their indices
   __shared__ int s_cnt;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -129,7 +139,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   const int hk = h / (p.H / p.Hkv);
   const int64_t bhk = (int64_t)b * p.Hkv + hk;
 
-  // ---- compact list of kept k-blocks ------------------------------------------------------
+  // ---- compact list of kept k-blocks (and of their k scales) ------------------------------
+  const float* ksc_base = p.k_scale + bhk * p.nbk;
   const int kmax = CAUSAL ? min(p.nbk, qb + 1) : p.nbk;
   if (wave == 0) {
     const uint8_t* mrow = p.sparse + b * p.sparse_bs + ((int64_t)h * p.nbq + qb) * p.nbk;
@@ -145,13 +156,20 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
       for (int u = 0; u < 4; u++) {
         const bool keep = m[u] != 0;
         const unsigned long long bal = __ballot(keep);
-        if (keep) klist[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (unsigned short)(base + u * 64 + lane);
+        if (keep) {
+          const int pos = cnt + __popcll(bal & ((1ull << lane) - 1ull));
+          klist[pos] = (unsigned short)(base + u * 64 + lane);
+          clist[pos] = ksc_base[base + u * 64 + lane];
+        }
         cnt += __popcll(bal);
         if (bal) last = base + u * 64 + 63 - __clzll(bal);
       }
     }
     // the loop prefetches up to 3 blocks ahead without branching: pad with the last kept block
-    if (lane < 4) klist[cnt + lane] = (unsigned short)last;
+    if (lane < 4) {
+      klist[cnt + lane] = (unsigned short)last;
+      clist[cnt + lane] = ksc_base[last];
+    }
     if (lane == 0) s_cnt = cnt;
   }
 
@@ -165,7 +183,6 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
   }
   const float qsc = p.q_scale[((int64_t)b * p.H + h) * (p.nbq * 2) + qb * 2 + wave] * p.sm_scale_log2e;
-  const float* ksc_base = static_cast<const float*>(uniform_ptr(p.k_scale + bhk * p.nbk));
 
   __syncthreads();
   const int cnt = s_cnt;
@@ -228,13 +245,15 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   };
   // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns.  The accumulators start at the bit
   // pattern of 1.5*2^23: the int32 result then READS as the float 12582912 + S exactly
-  // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.
+  // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.  Two accumulator sets
+  // alternate: the product for block i+1 runs on the matrix cores while the VALU works through the
+  // softmax of block i.
   v16i magic;
 #pragma unroll
   for (int i = 0; i < 16; i++) magic[i] = S_MAGIC_BITS;
   asm volatile("" : "+v"(magic));  // keep the constant block resident instead of rebuilding it per block
-  v16i acc[2];
-  auto qk_mfma = [&]() {
+  v16i acc_a[2], acc_b[2];
+  auto qk_mfma = [&](v16i (&acc)[2]) {
 #pragma unroll
     for (int mt = 0; mt < 2; mt++) {
       acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[mt], qf[0], magic, 0, 0, 0);
@@ -243,7 +262,7 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
         acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[ks * 2 + mt], qf[ks], acc[mt], 0, 0, 0);
     }
   };
-  auto dump_s = [&](int kb) {
+  auto dump_s = [&](int kb, v16i (&acc)[2]) {
     if constexpr (DUMP) {
       if (p.s_dump) {
         int32_t* sd = p.s_dump + (((int64_t)b * p.H + h) * (p.nbq * 64) + qrow) * (int64_t)(p.nbk * 64) + kb * 64;
@@ -282,28 +301,28 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   load_tile(kb_1);
   store_tile(1);
   load_tile(kb_2);
-  float c_cur = qsc * ksc_base[kb_c];
+  float c_cur = qsc * clist[0];
   __syncthreads();
   read_k_frags(0);
-  qk_mfma();
-  dump_s(kb_c);
+  qk_mfma(acc_a);
+  dump_s(kb_c, acc_a);
 
-  // one block; stage_c holds its V tile, stage_1 the K tile of the next block, stage_2 receives
-  // the block after that
-  auto step = [&](int it, int SC, int stage_1, int stage_2) {
-    // -- LDS traffic of this iteration, issued up front: index of block it+3, V fragments of the
-    //    current block, K fragments of the next one
+  // One block: `acc` holds its S^T, `acc_n` receives that of the next block.  stage_c holds the V
+  // tile of this block, stage_1 the K tile of the next one, stage_2 receives the block after that.
+  auto step = [&](int it, int stage_c, int stage_1, int stage_2, v16i (&acc)[2], v16i (&acc_n)[2]) {
+    // -- LDS traffic of this iteration, issued up front: index of block it+3, K fragments of the
+    //    next block, V fragments of this one
     const int kidx_v = (int)klist[it + 3];
+    read_k_frags(stage_1);
     v4i vfrag[DT_TILES][2];
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
       for (int mt = 0; mt < 2; mt++)
-        vfrag[dt][mt] = *reinterpret_cast<const v4i*>(smem + SC * Lds::VTILE + vr_base + (dt * 2 + mt) * 1024);
-    read_k_frags(stage_1);
-    const float c_next = qsc * ksc_base[kb_1];
+        vfrag[dt][mt] = *reinterpret_cast<const v4i*>(smem + stage_c * Lds::VTILE + vr_base + (dt * 2 + mt) * 1024);
+    const float c_next = qsc * clist[it + 1];
 
-    // -- softmax of the current block
+    // -- row maximum of this block (covers the LDS latency of the K fragments)
     float s[2][16];
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
@@ -323,17 +342,27 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
         }
     }
 
-    // two interleaved v_max3 chains (the values are integers read as floats: no NaN to canonicalise)
-    float mx0 = s[0][0], mx1 = s[1][0];
+    // four interleaved v_max3 chains (the values are integers read as floats: no NaN to canonicalise)
+    float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[0][8], s[0][9], s[0][10]);
+    float mx2 = max3(s[1][0], s[1][1], s[1][2]), mx3 = max3(s[1][8], s[1][9], s[1][10]);
 #pragma unroll
-    for (int i = 1; i < 15; i += 2) {
+    for (int i = 3; i < 7; i += 2) {
       mx0 = max3(mx0, s[0][i], s[0][i + 1]);
-      mx1 = max3(mx1, s[1][i], s[1][i + 1]);
+      mx1 = max3(mx1, s[0][i + 8], s[0][i + 9]);
+      mx2 = max3(mx2, s[1][i], s[1][i + 1]);
+      mx3 = max3(mx3, s[1][i + 8], s[1][i + 9]);
     }
-    float smax = max3(mx0, mx1, s[0][15]);
-    smax = max3(smax, s[1][15], smax);
-    smax = partner_max(smax) - S_MAGIC_F;  // exact: both are integers below 2^24
+    mx0 = max3(mx0, s[0][7], s[0][15]);
+    mx2 = max3(mx2, s[1][7], s[1][15]);
+    float smax = max3(mx0, mx1, mx2);
+    smax = max3(smax, mx3, mx3);
 
+    // -- S^T of the NEXT block goes to the matrix cores now and runs under the exponentials below
+    __builtin_amdgcn_sched_barrier(0);
+    qk_mfma(acc_n);
+    __builtin_amdgcn_sched_barrier(0);
+
+    smax = partner_max(smax) - S_MAGIC_F;  // exact: both are integers below 2^24
     const float c = c_cur;
     const float m_blk = smax * c;
     if (__ballot(m_blk > m_i + P_HEADROOM) != 0ull) {  // rare after the first few blocks
@@ -347,29 +376,51 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
     }
-    const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
-
     v8i pf;
     float rs = 0.f;
+    if constexpr (EXACT) {
+      // P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential, then the packed FP8 conversion
+      const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
 #pragma unroll
-    for (int r = 0; r < 8; r++) {
-      const int mt = r >> 2, i0 = 4 * (r & 3);
-      const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
-      const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
-      const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
-      const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
-      if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
-      int w;
-      cvt_pk_fp8<false>(w, p0, p1);
-      cvt_pk_fp8<true>(w, p2, p3);
-      pf[r] = w;
+      for (int r = 0; r < 8; r++) {
+        const int mt = r >> 2, i0 = 4 * (r & 3);
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
+        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
+        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
+        if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
+        int w;
+        cvt_pk_fp8<false>(w, p0, p1);
+        cvt_pk_fp8<true>(w, p2, p3);
+        pf[r] = w;
+      }
+    } else {
+      // The e4m3 byte of 2^t is built directly: byte = rne(8*(t + 7) + FAST_EXP_SHIFT), i.e. exponent
+      // field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of two
+      // (at most 6 % off, shifted to be centred).  One fma and one byte conversion per element
+      // instead of fma + v_exp_f32 + half a packed FP8 conversion; v_cvt_pk_u8_f32 rounds to nearest
+      // even and clamps to [0, 255], which sends masked (-inf) and underflowing elements to 0.
+      const float c8 = 8.0f * c;
+      const float bias8 = fmaf(-S_MAGIC_F, c8, 8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT);
+      // byte-major order: the four conversions into one word depend on each other, the eight words
+      // do not
+      int w[8];
+#pragma unroll
+      for (int r = 0; r < 8; r++) cvt_pk_u8<0, true>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 0], c8, bias8));
+#pragma unroll
+      for (int r = 0; r < 8; r++) cvt_pk_u8<1, false>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 1], c8, bias8));
+#pragma unroll
+      for (int r = 0; r < 8; r++) cvt_pk_u8<2, false>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 2], c8, bias8));
+#pragma unroll
+      for (int r = 0; r < 8; r++) cvt_pk_u8<3, false>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 3], c8, bias8));
+#pragma unroll
+      for (int r = 0; r < 8; r++) pf[r] = w[r];
     }
     if constexpr (LSE) d_exact += rs;
 
-    // -- S^T of the NEXT block first (its softmax opens the next iteration), then
-    //    O^T += V8^T . P~^T of this one; the row sums of the ROUNDED P~ come from one more MFMA
-    //    against ones
-    qk_mfma();
+    // -- O^T += V8^T . P~^T; the row sums of the ROUNDED P~ come from one more MFMA against ones.
+    //    These run under the barrier and the row maximum of the next iteration.
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; dt++) {
       const v8i a = {vfrag[dt][0][0], vfrag[dt][0][1], vfrag[dt][0][2], vfrag[dt][0][3],
@@ -377,21 +428,30 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
       o_acc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf, o_acc[dt], 0, 0, 0, 0, 0, 0);
     }
     d_acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
-    if (it + 1 < cnt) dump_s(kb_1);
+    __builtin_amdgcn_sched_barrier(0);
+    if (it + 1 < cnt) dump_s(kb_1, acc_n);
 
     // -- block it+2 from registers into the ring, block it+3 from HBM/L2 into registers
+#ifndef EXP_NOSTORE
     store_tile(stage_2);
+#endif
     const int kb_3 = __builtin_amdgcn_readfirstlane(kidx_v);
+#ifndef EXP_NOLOAD
     load_tile(kb_3);
+#endif
+#ifndef EXP_NOBARRIER
     __syncthreads();
+#endif
     kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3;
     c_cur = c_next;
   };
 
   int st_c = 0, st_1 = 1, st_2 = 2;
-  for (int it = 0; it < cnt; it++) {
-    step(it, st_c, st_1, st_2);
-    const int st_t = st_c; st_c = st_1; st_1 = st_2; st_2 = st_t;
+  for (int it = 0; it < cnt; it += 2) {
+    step(it, st_c, st_1, st_2, acc_a, acc_b);
+    if (it + 1 >= cnt) break;
+    step(it + 1, st_1, st_2, st_c, acc_b, acc_a);
+    const int st_t = st_c; st_c = st_2; st_2 = st_1; st_1 = st_t;
   }
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------
@@ -424,11 +484,11 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   }
 }
 
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE>
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
   const int grid = ((p.total + 7) / 8) * 8;
-  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + 4) * 2 + 15) & ~(size_t)15);
-  auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE>;
+  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + 4) * 6 + 15) & ~(size_t)15);
+  auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
   if (smem > 48 * 1024)
     PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(128), smem, st, p);
@@ -437,14 +497,19 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
 }
 
 template <int D, int OUT_DT>
-static int dispatch_attn(const AttnParams& p, int is_causal, bool dump, hipStream_t st) {
-  const bool lse = p.lse != nullptr;
-  if (dump) {  // debug path: one instantiation per causal mode, always with the exact row sum
-    if (is_causal) return launch_attn<D, OUT_DT, true, true, true>(p, st);
-    return launch_attn<D, OUT_DT, false, true, true>(p, st);
+static int dispatch_attn(const AttnParams& p, int is_causal, bool dump, bool exact, hipStream_t st) {
+  // the log-sum-exp needs true exponentials; the debug dump rides on the same instantiation
+  if (p.lse != nullptr || dump) {
+    if (dump) return is_causal ? launch_attn<D, OUT_DT, true, true, true, true>(p, st)
+                               : launch_attn<D, OUT_DT, false, true, true, true>(p, st);
+    return is_causal ? launch_attn<D, OUT_DT, true, false, true, true>(p, st)
+                     : launch_attn<D, OUT_DT, false, false, true, true>(p, st);
   }
-  if (is_causal) return lse ? launch_attn<D, OUT_DT, true, false, true>(p, st) : launch_attn<D, OUT_DT, true, false, false>(p, st);
-  return lse ? launch_attn<D, OUT_DT, false, false, true>(p, st) : launch_attn<D, OUT_DT, false, false, false>(p, st);
+  if (exact)
+    return is_causal ? launch_attn<D, OUT_DT, true, false, false, true>(p, st)
+                     : launch_attn<D, OUT_DT, false, false, false, true>(p, st);
+  return is_causal ? launch_attn<D, OUT_DT, true, false, false, false>(p, st)
+                   : launch_attn<D, OUT_DT, false, false, false, false>(p, st);
 }
 
 }  // namespace paro
@@ -455,8 +520,9 @@ extern "C" int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const ui
                                     float* lse, int32_t* s_dump, int B, int H, int Hkv, int Nq, int Nk, int D,
                                     int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
                                     int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
-                                    int64_t o_stride_n, float sm_scale, int is_causal, void* stream) {
+                                    int64_t o_stride_n, float sm_scale, int is_causal, int flags, void* stream) {
   using namespace paro;
+  PARO_CHECK((flags & ~PARO_ATTN_EXACT_EXP) == 0, PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
   PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && v_scale && sparse && out, PARO_ERR_RUNTIME,
              "paro_attn_sparse_fwd: null tensor pointer");
   PARO_CHECK(B > 0 && H > 0 && Hkv > 0 && Nq > 0 && Nk > 0, PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: empty shape");
@@ -488,12 +554,13 @@ extern "C" int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const ui
   p.sm_scale_log2e = sm_scale * 1.4426950408889634f;
   hipStream_t st = (hipStream_t)stream;
   const bool dump = s_dump != nullptr;
+  const bool exact = (flags & PARO_ATTN_EXACT_EXP) != 0;
   if (D == 64) {
-    if (out_dtype == PARO_DTYPE_F16) return dispatch_attn<64, PARO_DTYPE_F16>(p, is_causal, dump, st);
-    return dispatch_attn<64, PARO_DTYPE_BF16>(p, is_causal, dump, st);
+    if (out_dtype == PARO_DTYPE_F16) return dispatch_attn<64, PARO_DTYPE_F16>(p, is_causal, dump, exact, st);
+    return dispatch_attn<64, PARO_DTYPE_BF16>(p, is_causal, dump, exact, st);
   }
-  if (out_dtype == PARO_DTYPE_F16) return dispatch_attn<128, PARO_DTYPE_F16>(p, is_causal, dump, st);
-  return dispatch_attn<128, PARO_DTYPE_BF16>(p, is_causal, dump, st);
+  if (out_dtype == PARO_DTYPE_F16) return dispatch_attn<128, PARO_DTYPE_F16>(p, is_causal, dump, exact, st);
+  return dispatch_attn<128, PARO_DTYPE_BF16>(p, is_causal, dump, exact, st);
 }
 
 extern "C" int64_t paro_attn_workspace_bytes(int B, int Hkv, int Nk, int D) {
@@ -511,7 +578,7 @@ extern "C" int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, cons
                                         int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
                                         int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
                                         int tensor_layout, int is_causal, int qk_quant_gran, float sm_scale,
-                                        int smooth_v, void* stream) {
+                                        int smooth_v, int flags, void* stream) {
   using namespace paro;
   PARO_CHECK(tensor_layout == 0 || tensor_layout == 1, PARO_ERR_INVALID_VALUE, "tensor_layout must be 0 or 1");
   PARO_CHECK(qk_quant_gran == 2 || qk_quant_gran == 3, PARO_ERR_INVALID_VALUE, "Unsupported quantization granularity: %d",
@@ -540,5 +607,5 @@ extern "C" int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, cons
   return paro_attn_sparse_fwd(q8, k8, v8, q_scale, k_scale, v_scale, smooth_v ? v_mean : nullptr, sparse,
                               sparse_batch_stride, out, out_dtype, lse, nullptr, B, H, Hkv, Nq, Nk, D, q_stride_b,
                               q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n, o_stride_b, o_stride_h,
-                              o_stride_n, sm_scale, is_causal, stream);
+                              o_stride_n, sm_scale, is_causal, flags, stream);
 }

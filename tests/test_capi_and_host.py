@@ -61,15 +61,15 @@ def test_c_abi_argument_errors_without_gpu():
     rc = lib.paro_permute_inv(p, p, 0, p, 1, 1, 100, 64, 10, 3, 5, 7, 0, 0, 64, 0, 0, 64, None)
     assert rc == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
     rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
-                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 3, 0.125, 1, None)
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 3, 0.125, 1, 0, None)
     assert rc == L.PARO_ERR_UNSUPPORTED
     with pytest.raises(NotImplementedError):
         L.check(rc)
     rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 16, 1, 1, 1, 64, 64, 64,
-                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 2, 0.125, 1, None)
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 2, 0.125, 1, 0, None)
     assert rc == L.PARO_ERR_RUNTIME and b"workspace" in lib.paro_last_error()
     rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
-                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 7, 0, 2, 0.125, 1, None)
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 7, 0, 2, 0.125, 1, 0, None)
     assert rc == L.PARO_ERR_INVALID_VALUE and lib.paro_last_error() == b"tensor_layout must be 0 or 1"
 
 

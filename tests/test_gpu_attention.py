@@ -17,7 +17,7 @@ COS = 0.999
 
 
 def _run(dev, B, H, N, D, dtype, density, seed, Hkv=None, causal=False, smooth_k=True, return_lse=True,
-         mask=None, batch_mask=False):
+         mask=None, batch_mask=False, exact_exp=False):
     import paroatten_amd as P
     Hkv = Hkv or H
     q, _, _ = synth.make_qkv(B, H, N, D, dtype, seed=seed)
@@ -31,7 +31,7 @@ def _run(dev, B, H, N, D, dtype, density, seed, Hkv=None, causal=False, smooth_k
     o_ref, lse_ref = O.sparse_attention(q8, k8, v, qs, ks, mask_b, D ** -0.5, is_causal=causal, out_dtype=dtype)
     m_dev = (mask_b if batch_mask else mask).to(dev)
     out = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), m_dev, is_causal=causal,
-                                          smooth_k=smooth_k, return_lse=return_lse)
+                                          smooth_k=smooth_k, return_lse=return_lse, exact_exp=exact_exp)
     o, lse = out if return_lse else (out, None)
     return o.cpu(), (None if lse is None else lse.cpu()), o_ref, lse_ref / O.LOG2E, mask_b
 
@@ -49,12 +49,20 @@ def _assert_close(o, o_ref, baseline_shape=False):
 
 
 def test_cfg0_plumbing(dev):
-    """BASELINE config 0: B=1,H=2,D=64,fp16,N=4096, density 0.5, K bias."""
+    """BASELINE config 0: B=1,H=2,D=64,fp16,N=4096, density 0.5, K bias.  With lse the kernel
+    evaluates exact exponentials; without, its default fast path builds the e4m3 weights directly."""
     o, lse, o_ref, lse_ref, _ = _run(dev, 1, 2, 4096, 64, torch.float16, 0.5, seed=0)
     _assert_close(o, o_ref, baseline_shape=True)
     assert torch.allclose(lse, lse_ref, atol=2e-3, rtol=1e-4)
     for h in range(2):
         assert cosine(o[:, h], o_ref[:, h]) >= COS
+    for exact in (False, True):
+        o2, _, o_ref2, _, _ = _run(dev, 1, 2, 4096, 64, torch.float16, 0.5, seed=0, return_lse=False,
+                                   exact_exp=exact)
+        _assert_close(o2, o_ref2, baseline_shape=True)
+        for h in range(2):
+            assert cosine(o2[:, h], o_ref2[:, h]) >= COS
+    assert torch.equal(o2, o)  # exact_exp without lse == the lse instantiation
 
 
 @pytest.mark.parametrize("D,dtype", [(64, torch.bfloat16), (128, torch.float16), (128, torch.bfloat16)])
@@ -63,13 +71,17 @@ def test_shapes_and_tails(dev, D, dtype, N):
     o, lse, o_ref, lse_ref, _ = _run(dev, 2, 3, N, D, dtype, 0.4, seed=N + D, batch_mask=(N == 1000))
     _assert_close(o, o_ref)
     assert torch.allclose(lse, lse_ref, atol=2e-3, rtol=1e-4)
+    o, _, o_ref, _, _ = _run(dev, 2, 3, N, D, dtype, 0.4, seed=N + D, batch_mask=(N == 1000), return_lse=False)
+    _assert_close(o, o_ref)  # default fast exponential
 
 
 def test_dense_equals_masked_all_true(dev):
     nb = 9
     mask = torch.ones(2, nb, nb, dtype=torch.bool)
-    o, lse, o_ref, lse_ref, _ = _run(dev, 1, 2, 64 * nb - 13, 64, torch.float16, 1.0, seed=4, mask=mask)
-    _assert_close(o, o_ref)
+    for lse_on in (True, False):
+        o, lse, o_ref, lse_ref, _ = _run(dev, 1, 2, 64 * nb - 13, 64, torch.float16, 1.0, seed=4, mask=mask,
+                                         return_lse=lse_on)
+        _assert_close(o, o_ref)
 
 
 def test_empty_rows_and_single_block(dev):
@@ -96,6 +108,9 @@ def test_causal_and_gqa(dev):
                                      mask=torch.ones(4, 11, 11, dtype=torch.bool))
     _assert_close(o, o_ref)
     assert torch.allclose(lse, lse_ref, atol=2e-3, rtol=1e-4)
+    o, _, o_ref, _, _ = _run(dev, 1, 4, 700, 64, torch.float16, 1.0, seed=12, Hkv=2, causal=True,
+                             mask=torch.ones(4, 11, 11, dtype=torch.bool), return_lse=False)
+    _assert_close(o, o_ref)
 
 
 def test_no_smoothing_paths(dev):
@@ -143,7 +158,7 @@ def test_int32_qk_accumulators_bitexact(dev, D):
         L.ptr(q8d), L.ptr(k8d), L.ptr(v8), L.ptr(qsd), L.ptr(ksd), L.ptr(vsc), L.ptr(vm), L.ptr(md), md.stride(0),
         L.ptr(out), 0, None, L.ptr(dump), B, H, H, N, N, D,
         q8d.stride(0), q8d.stride(1), q8d.stride(2), k8d.stride(0), k8d.stride(1), k8d.stride(2),
-        out.stride(0), out.stride(1), out.stride(2), D ** -0.5, 0, L.stream_of(out)))
+        out.stride(0), out.stride(1), out.stride(2), D ** -0.5, 0, 0, L.stream_of(out)))
     dump = dump.cpu()
     keep = O.expand_block_mask(mask, nb * 64, nb * 64)
     # computed blocks: exact on the real rows/columns; skipped blocks: untouched
