@@ -106,12 +106,26 @@ __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, int vo
 }
 
 template <int D> struct AttnLds {
-  static constexpr int KPITCH = D + 16;        // padded K rows: conflict-free 16-byte column reads
-  static constexpr int KTILE = 64 * KPITCH;    // bytes of one K8 tile in LDS
-  static constexpr int VTILE = 64 * D;         // bytes of one V8 tile (fragment order, as in HBM)
+  static constexpr int KTILE = 64 * D;   // bytes of one K8 tile: 64 rows of D bytes, 16-byte chunks XOR-swizzled
+  static constexpr int VTILE = 64 * D;   // bytes of one V8 tile (fragment order, as in HBM)
   static constexpr int V_OFF = NST * KTILE;
   static constexpr int LIST_OFF = NST * (KTILE + VTILE);
+  static constexpr int LIST_PAD = 8;     // list entries past the end that the prefetch may touch
+  // chunk c of row `row` is stored at chunk position c ^ swz(row): makes the MFMA A-operand reads (32
+  // rows x one 16-byte chunk per half-wave) conflict-free; measured on gfx950 for both row lengths
+  static __device__ __forceinline__ int swz(int row) {
+    if constexpr (D == 64) return (row >> 2) & 3;
+    else return (row ^ (row >> 3)) & 7;
+  }
 };
+
+// LDS-DMA: 16 bytes per lane from a buffer straight into LDS at lds_base + lane*16; no registers, no
+// ds_write; completion is counted by vmcnt
+__device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_base, int voffset,
+                                                  int soffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_base, 16, voffset,
+                                           soffset, 0, 0);
+}
 
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p) {
@@ -122,8 +136,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* clist = reinterpret_cast<float*>(smem + Lds::LIST_OFF);                       // [nbk + 4] k_scale of kept blocks
-  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + p.nbk + 4);  // [nbk + 4] their indices
+  float* clist = reinterpret_cast<float*>(smem + Lds::LIST_OFF);  // [nbk + LIST_PAD] k_scale of kept blocks
+  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + p.nbk + Lds::LIST_PAD);  // their indices
   __shared__ int s_cnt;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -165,8 +179,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
         if (bal) last = base + u * 64 + 63 - __clzll(bal);
       }
     }
-    // the loop prefetches up to 3 blocks ahead without branching: pad with the last kept block
-    if (lane < 4) {
+    // the loop prefetches up to 4 blocks ahead without branching: pad with the last kept block
+    if (lane < Lds::LIST_PAD) {
       klist[cnt + lane] = (unsigned short)last;
       clist[cnt + lane] = ksc_base[last];
     }
@@ -199,70 +213,72 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     return;
   }
 
-  // ---- tile movers: buffer loads (scalar base + per-thread offset fixed for the whole loop +
-  //      scalar per-block offset), staged through registers into the LDS ring ------------------
+  // ---- tile movers: LDS-DMA buffer loads (scalar base + per-lane offset fixed for the whole loop +
+  //      scalar per-block offset).  Each wave moves half of every tile, 1 KB (64 lanes x 16 bytes) per
+  //      instruction; K8's chunk swizzle is applied on the global-address side. ---------------------
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr(p.k8 + b * p.ks_b + hk * p.ks_h), 0, (int)((int64_t)(p.Nk - 1) * p.ks_n + D), 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr(p.v8 + bhk * p.nbk * (int64_t)Lds::VTILE), 0, p.nbk * Lds::VTILE, 0x00020000);
-  int k_goff[NLD], k_loff[NLD], v_off[NLD];
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  int k_goff[NLD], v_goff[NLD];
 #pragma unroll
   for (int i = 0; i < NLD; i++) {
-    const int c = t + 128 * i;
-    const int row = c / CPR, cc = c % CPR;
-    k_goff[i] = row * (int)p.ks_n + cc * 16;
-    k_loff[i] = row * Lds::KPITCH + cc * 16;
-    v_off[i] = c * 16;
+    const int pos = (wave_u * NLD + i) * 1024 + lane * 16;  // byte position inside the LDS tile
+    const int row = pos / D, cpos = (pos % D) / 16;
+    k_goff[i] = row * (int)p.ks_n + ((cpos ^ Lds::swz(row)) * 16);
+    v_goff[i] = pos;
   }
   const int k_blk_stride = 64 * (int)p.ks_n;
-  v4i kst[NLD], vst[NLD];
-  auto load_tile = [&](int kb) {
+  auto load_k = [&](int kb, int ST) {  // rows >= Nk read as 0
 #pragma unroll
-    for (int i = 0; i < NLD; i++) {
-      kst[i] = buffer_load16(k_rsrc, k_goff[i], kb * k_blk_stride);  // rows >= Nk read as 0
-      vst[i] = buffer_load16(v_rsrc, v_off[i], kb * Lds::VTILE);
-    }
+    for (int i = 0; i < NLD; i++)
+      buffer_load16_lds(k_rsrc, smem + ST * Lds::KTILE + (wave_u * NLD + i) * 1024, k_goff[i], kb * k_blk_stride);
   };
-  auto store_tile = [&](int ST) {
+  auto load_v = [&](int kb, int ST) {
 #pragma unroll
-    for (int i = 0; i < NLD; i++) {
-      *reinterpret_cast<v4i*>(smem + ST * Lds::KTILE + k_loff[i]) = kst[i];
-      *reinterpret_cast<v4i*>(smem + Lds::V_OFF + ST * Lds::VTILE + v_off[i]) = vst[i];
-    }
+    for (int i = 0; i < NLD; i++)
+      buffer_load16_lds(v_rsrc, smem + Lds::V_OFF + ST * Lds::VTILE + (wave_u * NLD + i) * 1024, v_goff[i],
+                        kb * Lds::VTILE);
   };
+  constexpr int LOADS_PER_IT = 2 * NLD;  // DMA instructions one wave issues per block
 
   // ---- fragment movers and the two matrix products ---------------------------------------
-  const int kr_base = l32 * Lds::KPITCH + lh * 16;  // K fragment (ks, mt): + ks*32 + mt*32*KPITCH
   const int vr_base = Lds::V_OFF + lane * 16;        // V fragment (dt, mt): + (dt*2+mt)*1024
   v4i kfrag[2 * KS];
+  // K fragment (ks, mt): row 32*mt + l32, chunk 2*ks + lh at its swizzled position
+  int kr_off[2 * KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+    for (int mt = 0; mt < 2; mt++) {
+      const int row = 32 * mt + l32;
+      kr_off[ks * 2 + mt] = row * D + (((2 * ks + lh) ^ Lds::swz(row)) * 16);
+    }
   auto read_k_frags = [&](int ST) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-      for (int mt = 0; mt < 2; mt++)
-        kfrag[ks * 2 + mt] =
-            *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + kr_base + ks * 32 + mt * 32 * Lds::KPITCH);
+    for (int i = 0; i < 2 * KS; i++) kfrag[i] = *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + kr_off[i]);
   };
   // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns.  The accumulators start at the bit
   // pattern of 1.5*2^23: the int32 result then READS as the float 12582912 + S exactly
-  // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.  Two accumulator sets
-  // alternate: the product for block i+1 runs on the matrix cores while the VALU works through the
-  // softmax of block i.
+  // (|S| <= 127*127*128 < 2^22), which saves the int->float conversions.
   v16i magic;
 #pragma unroll
   for (int i = 0; i < 16; i++) magic[i] = S_MAGIC_BITS;
   asm volatile("" : "+v"(magic));  // keep the constant block resident instead of rebuilding it per block
-  v16i acc_a[2], acc_b[2];
-  auto qk_mfma = [&](v16i (&acc)[2]) {
-#pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
-      acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[mt], qf[0], magic, 0, 0, 0);
-#pragma unroll
-      for (int ks = 1; ks < KS; ks++)
-        acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[ks * 2 + mt], qf[ks], acc[mt], 0, 0, 0);
-    }
+  v16i acc[2];
+  // the MFMAs are issued one at a time from inside the VALU stream (see step below): a wave that
+  // issues them back to back sits blocked behind the matrix pipe for their whole duration
+  auto qk_one = [&](int idx) {  // idx = mt * KS + ks, ks ascending per mt
+    const int mt = idx / KS, ks = idx % KS;
+    if (ks == 0) acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[mt], qf[0], magic, 0, 0, 0);
+    else acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[ks * 2 + mt], qf[ks], acc[mt], 0, 0, 0);
   };
-  auto dump_s = [&](int kb, v16i (&acc)[2]) {
+  auto qk_mfma = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2 * KS; i++) qk_one(i);
+  };
+  auto dump_s = [&](int kb) {
     if constexpr (DUMP) {
       if (p.s_dump) {
         int32_t* sd = p.s_dump + (((int64_t)b * p.H + h) * (p.nbq * 64) + qrow) * (int64_t)(p.nbk * 64) + kb * 64;
@@ -289,40 +305,66 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   float m_i = -1e30f;
   float d_exact = 0.f;  // LSE only: sum of the unrounded P~ of this lane's 32 kv-columns per block
 
-  // ---- prologue: blocks 0 and 1 into the ring, block 2 in flight, S of block 0 ---------------
-  using I0 = std::integral_constant<int, 0>;
-  using I1 = std::integral_constant<int, 1>;
-  using I2 = std::integral_constant<int, 2>;
+  // ---- prologue ------------------------------------------------------------------------------
+  // K ring: stage j%3 holds the K tile of block j; V ring likewise.  Block i's S^T is produced one
+  // iteration ahead of its softmax and its P.V one iteration behind:
+  //   iteration i:  DMA K(i+3), V(i+1) | reads K(i+1), V(i-1) | S(i+1) = K(i+1).Q | P(i) = softmax(S(i))
+  //                 | O += V(i-1).P(i-1)
+  // What iteration i issues is waited for at the end of iteration i+1 (vmcnt keeps the newest
+  // LOADS_PER_IT in flight) and published by that iteration's barrier.
   int kb_c = __builtin_amdgcn_readfirstlane((int)klist[0]);
   int kb_1 = __builtin_amdgcn_readfirstlane((int)klist[1]);
   int kb_2 = __builtin_amdgcn_readfirstlane((int)klist[2]);
-  load_tile(kb_c);
-  store_tile(0);
-  load_tile(kb_1);
-  store_tile(1);
-  load_tile(kb_2);
+  int kb_3 = __builtin_amdgcn_readfirstlane((int)klist[3]);
+  load_k(kb_c, 0);
+  load_v(kb_c, 0);
+  load_v(kb_c, 2);  // the first iteration multiplies this stage by an all-zero P: it must hold finite values
+  load_k(kb_1, 1);
+  load_k(kb_2, 2);
   float c_cur = qsc * clist[0];
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   read_k_frags(0);
-  qk_mfma(acc_a);
-  dump_s(kb_c, acc_a);
+  qk_mfma();
+  dump_s(kb_c);
+  v8i pf_a = {0, 0, 0, 0, 0, 0, 0, 0}, pf_b = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // One block: `acc` holds its S^T, `acc_n` receives that of the next block.  stage_c holds the V
-  // tile of this block, stage_1 the K tile of the next one, stage_2 receives the block after that.
-  auto step = [&](int it, int stage_c, int stage_1, int stage_2, v16i (&acc)[2], v16i (&acc_n)[2]) {
-    // -- LDS traffic of this iteration, issued up front: index of block it+3, K fragments of the
-    //    next block, V fragments of this one
-    const int kidx_v = (int)klist[it + 3];
-    read_k_frags(stage_1);
-    v4i vfrag[DT_TILES][2];
+  // the pending product O^T += V8^T(prev) . P~^T(prev), plus the row sums of the ROUNDED P~ from one
+  // more MFMA against ones; idx 0..DT_TILES-1 = output tiles, DT_TILES = row sums
+  v4i vfrag[DT_TILES][2];
+  auto pv_one = [&](const v8i& pf, int idx) {
+    if (idx < DT_TILES) {
+      const v8i a = {vfrag[idx][0][0], vfrag[idx][0][1], vfrag[idx][0][2], vfrag[idx][0][3],
+                     vfrag[idx][1][0], vfrag[idx][1][1], vfrag[idx][1][2], vfrag[idx][1][3]};
+      o_acc[idx] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf, o_acc[idx], 0, 0, 0, 0, 0, 0);
+    } else {
+      d_acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
+    }
+  };
+  auto read_v_frags = [&](int ST) {
 #pragma unroll
     for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
       for (int mt = 0; mt < 2; mt++)
-        vfrag[dt][mt] = *reinterpret_cast<const v4i*>(smem + stage_c * Lds::VTILE + vr_base + (dt * 2 + mt) * 1024);
+        vfrag[dt][mt] = *reinterpret_cast<const v4i*>(smem + ST * Lds::VTILE + vr_base + (dt * 2 + mt) * 1024);
+  };
+
+  constexpr int N_PV = DT_TILES + 1;     // MFMAs of one P.V (+ row sums)
+  // One block.  `acc` holds its S^T on entry and that of the next block on exit: row tile 0 is
+  // consumed by chunks 0-3 of the stream below and re-issued right after them, row tile 1 after the
+  // last chunk.  `pf` receives the block's P~, `pf_p` holds that of the previous block.  sk1: K stage
+  // of block it+1; svp/sv1: V stages of blocks it-1 / it+1; K(it+3) goes to the stage K(it) has just
+  // left (sk0).
+  auto step = [&](int it, int sk0, int sk1, int svp, int sv1, v8i& pf, v8i& pf_p) {
+    // -- memory traffic of this iteration, issued up front
+    load_k(kb_3, sk0);
+    load_v(kb_1, sv1);
+    const int kidx_v = (int)klist[it + 4];
+    read_k_frags(sk1);
+    read_v_frags(svp);
     const float c_next = qsc * clist[it + 1];
 
-    // -- row maximum of this block (covers the LDS latency of the K fragments)
+    // -- row maximum of this block
     float s[2][16];
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
@@ -356,102 +398,123 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     mx2 = max3(mx2, s[1][7], s[1][15]);
     float smax = max3(mx0, mx1, mx2);
     smax = max3(smax, mx3, mx3);
-
-    // -- S^T of the NEXT block goes to the matrix cores now and runs under the exponentials below
-    __builtin_amdgcn_sched_barrier(0);
-    qk_mfma(acc_n);
-    __builtin_amdgcn_sched_barrier(0);
-
     smax = partner_max(smax) - S_MAGIC_F;  // exact: both are integers below 2^24
+
     const float c = c_cur;
     const float m_blk = smax * c;
-    if (__ballot(m_blk > m_i + P_HEADROOM) != 0ull) {  // rare after the first few blocks
+    // Lazy refresh of the running maximum (rare after the first few blocks).  The new maximum
+    // applies to this block's weights at once; O and the row sums, which the pending P.V of the
+    // previous block still has to reach through the stream below, are rescaled after the stream.
+    const bool refresh = __ballot(m_blk > m_i + P_HEADROOM) != 0ull;
+    float alpha = 1.0f;
+    if (refresh) {
       const float m_new = fmaxf(m_i, m_blk);
-      const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+      alpha = __builtin_amdgcn_exp2f(m_i - m_new);
       m_i = m_new;
       if constexpr (LSE) d_exact *= alpha;
+    }
+
+    // -- the softmax weights of this block in 8 chunks (one 32-bit word of four e4m3 values each);
+    //    after each chunk one MFMA goes to the matrix pipe: first S^T of the NEXT block, then the
+    //    pending P.V of the PREVIOUS block.  All their operands are ready before the stream starts.
+    float rs = 0.f;
+    const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
+    const float c8 = 8.0f * c;
+    const float bias8 = fmaf(-S_MAGIC_F, c8, 8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT);
+    // MFMA issue plan: the pending P.V first (its operands are ready), S^T row tile 0 of the next
+    // block once chunk 3 has read the last of the current one, row tile 1 after chunk 7
+    auto mfma_after_chunk = [&](int r) {
+      if constexpr (D == 64) {
+        if (r < 3) pv_one(pf_p, r);
+        else if (r == 3) qk_one(0);
+        else if (r == 4) qk_one(1);
+        else if (r == 7) { qk_one(2); qk_one(3); }
+      } else {
+        if (r < 3) pv_one(pf_p, r);
+        else if (r == 3) { pv_one(pf_p, 3); pv_one(pf_p, 4); qk_one(0); }
+        else if (r == 4) qk_one(1);
+        else if (r == 5) qk_one(2);
+        else if (r == 6) qk_one(3);
+        else { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
+      }
+    };
+    // Fast path: the e4m3 byte of 2^t is built directly: byte = rne(8*(t + 7) + FAST_EXP_SHIFT), i.e.
+    // exponent field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of
+    // two (at most 6 % off, shifted to be centred).  One fma and one byte conversion per element
+    // instead of fma + v_exp_f32 + half a packed FP8 conversion; v_cvt_pk_u8_f32 rounds to nearest
+    // even and clamps to [0, 255], which sends masked (-inf) and underflowing elements to 0.  Its
+    // chunk r = (row tile r/4, byte r%4 of that tile's four words): the four conversions of a chunk
+    // are independent of each other.
+    int wf[8];
+#pragma unroll
+    for (int r = 0; r < 8; r++) {
+      const int mt = r >> 2, i0 = 4 * (r & 3);
+      int w;
+      if constexpr (!EXACT) {
+        const int byte = r & 3;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const float u = fmaf(s[mt][4 * q + byte], c8, bias8);
+          if (byte == 0) cvt_pk_u8<0, true>(wf[mt * 4 + q], u);
+          else if (byte == 1) cvt_pk_u8<1, false>(wf[mt * 4 + q], u);
+          else if (byte == 2) cvt_pk_u8<2, false>(wf[mt * 4 + q], u);
+          else cvt_pk_u8<3, false>(wf[mt * 4 + q], u);
+        }
+      } else {
+        // P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential, then the packed FP8 conversion
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
+        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
+        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
+        if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
+        cvt_pk_fp8<false>(w, p0, p1);
+        cvt_pk_fp8<true>(w, p2, p3);
+      }
+      if constexpr (EXACT) pf[r] = w;
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_after_chunk(r);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (!EXACT) {
+#pragma unroll
+      for (int r = 0; r < 8; r++) pf[r] = wf[r];
+    }
+    if constexpr (LSE) d_exact += rs;
+    if (it + 1 < cnt) dump_s(kb_1);
+    if (refresh) {
       d_acc[0] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
     }
-    v8i pf;
-    float rs = 0.f;
-    if constexpr (EXACT) {
-      // P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential, then the packed FP8 conversion
-      const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
-#pragma unroll
-      for (int r = 0; r < 8; r++) {
-        const int mt = r >> 2, i0 = 4 * (r & 3);
-        const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
-        const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
-        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
-        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
-        if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
-        int w;
-        cvt_pk_fp8<false>(w, p0, p1);
-        cvt_pk_fp8<true>(w, p2, p3);
-        pf[r] = w;
-      }
-    } else {
-      // The e4m3 byte of 2^t is built directly: byte = rne(8*(t + 7) + FAST_EXP_SHIFT), i.e. exponent
-      // field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of two
-      // (at most 6 % off, shifted to be centred).  One fma and one byte conversion per element
-      // instead of fma + v_exp_f32 + half a packed FP8 conversion; v_cvt_pk_u8_f32 rounds to nearest
-      // even and clamps to [0, 255], which sends masked (-inf) and underflowing elements to 0.
-      const float c8 = 8.0f * c;
-      const float bias8 = fmaf(-S_MAGIC_F, c8, 8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT);
-      // byte-major order: the four conversions into one word depend on each other, the eight words
-      // do not
-      int w[8];
-#pragma unroll
-      for (int r = 0; r < 8; r++) cvt_pk_u8<0, true>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 0], c8, bias8));
-#pragma unroll
-      for (int r = 0; r < 8; r++) cvt_pk_u8<1, false>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 1], c8, bias8));
-#pragma unroll
-      for (int r = 0; r < 8; r++) cvt_pk_u8<2, false>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 2], c8, bias8));
-#pragma unroll
-      for (int r = 0; r < 8; r++) cvt_pk_u8<3, false>(w[r], fmaf(s[r >> 2][4 * (r & 3) + 3], c8, bias8));
-#pragma unroll
-      for (int r = 0; r < 8; r++) pf[r] = w[r];
-    }
-    if constexpr (LSE) d_exact += rs;
 
-    // -- O^T += V8^T . P~^T; the row sums of the ROUNDED P~ come from one more MFMA against ones.
-    //    These run under the barrier and the row maximum of the next iteration.
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int dt = 0; dt < DT_TILES; dt++) {
-      const v8i a = {vfrag[dt][0][0], vfrag[dt][0][1], vfrag[dt][0][2], vfrag[dt][0][3],
-                     vfrag[dt][1][0], vfrag[dt][1][1], vfrag[dt][1][2], vfrag[dt][1][3]};
-      o_acc[dt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf, o_acc[dt], 0, 0, 0, 0, 0, 0);
-    }
-    d_acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (it + 1 < cnt) dump_s(kb_1, acc_n);
-
-    // -- block it+2 from registers into the ring, block it+3 from HBM/L2 into registers
-#ifndef EXP_NOSTORE
-    store_tile(stage_2);
-#endif
-    const int kb_3 = __builtin_amdgcn_readfirstlane(kidx_v);
-#ifndef EXP_NOLOAD
-    load_tile(kb_3);
-#endif
-#ifndef EXP_NOBARRIER
+    // -- everything the PREVIOUS iteration sent to LDS has to have landed before the barrier
+    //    publishes it; this iteration's own DMA may stay in flight
+    const int kb_4 = __builtin_amdgcn_readfirstlane(kidx_v);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS_PER_IT) : "memory");
     __syncthreads();
-#endif
-    kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3;
+    kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3; kb_3 = kb_4;
     c_cur = c_next;
   };
 
-  int st_c = 0, st_1 = 1, st_2 = 2;
+  // stage of block j is j % 3: with i = it % 3 the step writes K stage i, reads K stage i+1, reads V
+  // stage i-1 and writes V stage i+1
+  int i3 = 0;  // it % 3
   for (int it = 0; it < cnt; it += 2) {
-    step(it, st_c, st_1, st_2, acc_a, acc_b);
-    if (it + 1 >= cnt) break;
-    step(it + 1, st_1, st_2, st_c, acc_b, acc_a);
-    const int st_t = st_c; st_c = st_2; st_2 = st_1; st_1 = st_t;
+    const int s1 = i3 == 2 ? 0 : i3 + 1, s2 = i3 == 0 ? 2 : i3 - 1;  // (i3+1)%3, (i3+2)%3 == (i3-1)%3
+    step(it, i3, s1, s2, s1, pf_a, pf_b);
+    if (it + 1 >= cnt) { i3 = s1; break; }
+    step(it + 1, s1, s2, i3, s2, pf_b, pf_a);
+    i3 = s2;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // DMA of the padded tail blocks: nobody reads it
+  // the last block's P.V is still pending: i3 is now cnt % 3, its V tile sits in stage (cnt-1) % 3
+  {
+    read_v_frags(i3 == 0 ? 2 : i3 - 1);
+    const v8i& pf_last = (cnt & 1) ? pf_a : pf_b;
+#pragma unroll
+    for (int i = 0; i < N_PV; i++) pv_one(pf_last, i);
   }
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------
@@ -487,7 +550,7 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
   const int grid = ((p.total + 7) / 8) * 8;
-  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + 4) * 6 + 15) & ~(size_t)15);
+  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + AttnLds<D>::LIST_PAD) * 6 + 15) & ~(size_t)15);
   auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
   if (smem > 48 * 1024)
     PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
