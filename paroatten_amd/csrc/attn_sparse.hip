@@ -265,7 +265,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   v16i magic;
 #pragma unroll
   for (int i = 0; i < 16; i++) magic[i] = S_MAGIC_BITS;
-  asm volatile("" : "+v"(magic));  // keep the constant block resident instead of rebuilding it per block
+  // D = 64 has registers to spare: keep the constant block resident instead of rebuilding it per block
+  if constexpr (D == 64) asm volatile("" : "+v"(magic));
   v16i acc[2];
   // the MFMAs are issued one at a time from inside the VALU stream (see step below): a wave that
   // issues them back to back sits blocked behind the matrix pipe for their whole duration
@@ -446,20 +447,32 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     // chunk r = (row tile r/4, byte r%4 of that tile's four words): the four conversions of a chunk
     // are independent of each other.
     int wf[8];
+    float u_cur[4], u_nxt[4];
+    if constexpr (!EXACT) {
+#pragma unroll
+      for (int q = 0; q < 4; q++) u_cur[q] = fmaf(s[0][4 * q], c8, bias8);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int r = 0; r < 8; r++) {
       const int mt = r >> 2, i0 = 4 * (r & 3);
       int w;
       if constexpr (!EXACT) {
+        // the fmas of the next chunk are issued between this chunk's conversions: every conversion
+        // finds its input ready
         const int byte = r & 3;
+        const int rn = r + 1, mtn = rn >> 2, byten = rn & 3;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-          const float u = fmaf(s[mt][4 * q + byte], c8, bias8);
-          if (byte == 0) cvt_pk_u8<0, true>(wf[mt * 4 + q], u);
-          else if (byte == 1) cvt_pk_u8<1, false>(wf[mt * 4 + q], u);
-          else if (byte == 2) cvt_pk_u8<2, false>(wf[mt * 4 + q], u);
-          else cvt_pk_u8<3, false>(wf[mt * 4 + q], u);
+          if (rn < 8) u_nxt[q] = fmaf(s[mtn][4 * q + byten], c8, bias8);
+          if (byte == 0) cvt_pk_u8<0, true>(wf[mt * 4 + q], u_cur[q]);
+          else if (byte == 1) cvt_pk_u8<1, false>(wf[mt * 4 + q], u_cur[q]);
+          else if (byte == 2) cvt_pk_u8<2, false>(wf[mt * 4 + q], u_cur[q]);
+          else cvt_pk_u8<3, false>(wf[mt * 4 + q], u_cur[q]);
+          __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
       } else {
         // P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential, then the packed FP8 conversion
         const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
@@ -492,8 +505,9 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     // -- everything the PREVIOUS iteration sent to LDS has to have landed before the barrier
     //    publishes it; this iteration's own DMA may stay in flight
     const int kb_4 = __builtin_amdgcn_readfirstlane(kidx_v);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS_PER_IT) : "memory");
-    __syncthreads();
+    // (a bare s_barrier: __syncthreads() would add a fence that waits for ALL outstanding loads)
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS_PER_IT) : "memory");
+    __builtin_amdgcn_s_barrier();
     kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3; kb_3 = kb_4;
     c_cur = c_next;
   };
