@@ -34,8 +34,9 @@ PEAK_HBM_GBS = 8000.0
 HEADLINE_DENSITY = 0.3
 DENSITIES = (0.5, 0.3, 0.2)
 # HBM bytes per attention-kernel launch at density 0.3 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/attn_sparse_cogvideox5b_pmc.txt); None until measured
-ATTN_TRAFFIC_BYTES = None
+# (profiles/attn_sparse_cogvideox5b_pmc.txt): FETCH_SIZE 164683 x 2.0 KiB + WRITE_SIZE 213341 x 1.0 KiB,
+# the factors being what the same counters read for a plain copy of known size
+ATTN_TRAFFIC_BYTES = int((164683 * 2.0 + 213341 * 1.0) * 1024)
 
 
 def event_time_ms(fn, reps, warmup):
@@ -86,6 +87,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the headline density and the attention kernel: the run to put under a profiler")
     ap.add_argument("--workload", default="cogvideox5b", choices=["cogvideox5b", "wan14b_480p", "wan14b_720p"])
     args = ap.parse_args()
     if args.gpus != 1:
@@ -153,7 +156,7 @@ def main():
     # ---- per-density detail and the roofline of the attention kernel -------------------------
     reps = max(5, min(args.steps, 50))
     dens = {}
-    for d in DENSITIES:
+    for d in ((HEADLINE_DENSITY,) if args.headline_only else DENSITIES):
         t_entry = event_time_ms(lambda: entry(masks[d]), reps, 2)
         t_kern = event_time_ms(lambda: attn_only(masks[d]), reps, 2)
         ex_ops = synth.attention_ops(masks[d], D) * B
@@ -183,18 +186,19 @@ def main():
     # ---- the bandwidth-bound kernels of the path -------------------------------------------------
     el = B * H * N * D
     path = {}
-    t = event_time_ms(lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), reps, 2)
-    path["rope_permute_qkv"] = {"ms": round(t, 4), "GBps": round(3 * 2 * el * 2 / t / 1e6, 1)}
-    t = event_time_ms(lambda: PM.rope_permute(q, k, None, orders, wl.grid, wl.n_text, cos, sin), reps, 2)
-    path["rope_permute_qk"] = {"ms": round(t, 4), "GBps": round(2 * 2 * el * 2 / t / 1e6, 1)}
-    t = event_time_ms(lambda: PM.permute_inverse(out, orders, wl.grid, wl.n_text), reps, 2)
-    path["permute_inverse_o"] = {"ms": round(t, 4), "GBps": round(2 * el * 2 / t / 1e6, 1)}
-    t = event_time_ms(lambda: Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64), reps, 2)
-    path["quant_int8_qk"] = {"ms": round(t, 4), "GBps": round(2 * el * 3 / t / 1e6, 1)}
-    t = event_time_ms(lambda: Q.per_channel_fp8(vp), reps, 2)
-    path["v_fp8_pack"] = {"ms": round(t, 4), "GBps": round(el * 5 / t / 1e6, 1)}
-    for p in path.values():
-        p["frac_hbm_peak"] = round(p["GBps"] / PEAK_HBM_GBS, 3)
+    if not args.headline_only:
+        def timed(name, fn, nbytes):
+            t = event_time_ms(fn, reps, 2)
+            path[name] = {"ms": round(t, 4), "GBps": round(nbytes / t / 1e6, 1)}
+            path[name]["frac_hbm_peak"] = round(path[name]["GBps"] / PEAK_HBM_GBS, 3)
+
+        timed("rope_permute_qkv", lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), 3 * 2 * el * 2)
+        timed("rope_permute_qk", lambda: PM.rope_permute(q, k, None, orders, wl.grid, wl.n_text, cos, sin), 2 * 2 * el * 2)
+        timed("permute_inverse_o", lambda: PM.permute_inverse(out, orders, wl.grid, wl.n_text), 2 * el * 2)
+        timed("quant_int8_qk", lambda: Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64), 2 * el * 3)
+        timed("v_fp8_pack", lambda: Q.per_channel_fp8(vp), el * 5)
+        # plain device copy of one tensor: what this box sustains for the simplest read+write
+        timed("hbm_copy_reference", lambda: out.copy_(q), 2 * el * 2)
 
     result = {
         "metric": "effective attn TOPS & %MFMA peak @CogVideoX-5b shape, density 0.2/0.3/0.5",
