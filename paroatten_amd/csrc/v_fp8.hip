@@ -80,21 +80,37 @@ __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __re
 }
 
 template <int D>
-__global__ void v_finalize_kernel(const float* __restrict__ partial, float* __restrict__ v_scale,
-                                  float* __restrict__ v_mean, int N, int n_chunks, int smooth) {
-  const int t = threadIdx.x;
+__global__ void __launch_bounds__(1024) v_finalize_kernel(const float* __restrict__ partial,
+                                                          float* __restrict__ v_scale,
+                                                          float* __restrict__ v_mean, int N, int n_chunks,
+                                                          int smooth) {
+  // 1024 / D slices of the chunk range per channel, combined through LDS in a fixed order
+  constexpr int SL = 1024 / D;
+  __shared__ float red[3][SL][D];
+  const int ch = threadIdx.x % D, sl = threadIdx.x / D;
   const int64_t bh = blockIdx.x;
   const float* p = partial + bh * n_chunks * 3 * D;
   float s = 0.f, mn = INFINITY, mx = -INFINITY;
-  for (int c = 0; c < n_chunks; c++) {
-    s += p[(c * 3 + 0) * D + t];
-    mn = fminf(mn, p[(c * 3 + 1) * D + t]);
-    mx = fmaxf(mx, p[(c * 3 + 2) * D + t]);
+  for (int c = sl; c < n_chunks; c += SL) {
+    s += p[(c * 3 + 0) * D + ch];
+    mn = fminf(mn, p[(c * 3 + 1) * D + ch]);
+    mx = fmaxf(mx, p[(c * 3 + 2) * D + ch]);
   }
-  const float mean = smooth ? s / (float)N : 0.f;
-  const float amax = fmaxf(mx - mean, mean - mn);
-  v_scale[bh * D + t] = amax / 448.0f;
-  if (v_mean) v_mean[bh * D + t] = mean;
+  red[0][sl][ch] = s;
+  red[1][sl][ch] = mn;
+  red[2][sl][ch] = mx;
+  __syncthreads();
+  if (sl == 0) {
+    for (int i = 1; i < SL; i++) {
+      s += red[0][i][ch];
+      mn = fminf(mn, red[1][i][ch]);
+      mx = fmaxf(mx, red[2][i][ch]);
+    }
+    const float mean = smooth ? s / (float)N : 0.f;
+    const float amax = fmaxf(mx - mean, mean - mn);
+    v_scale[bh * D + ch] = amax / 448.0f;
+    if (v_mean) v_mean[bh * D + ch] = mean;
+  }
 }
 
 template <int DT, int D>
@@ -152,7 +168,7 @@ static int run_v_fp8(const void* v, uint8_t* v8, float* v_scale, float* v_mean, 
   hipLaunchKernelGGL((v_stats_kernel<DT, D>), dim3(n_chunks, Hkv, B), dim3(256), 0, st, vp, partial, N, n_chunks,
                      vs_b, vs_h, vs_n);
   PARO_HIP(hipGetLastError());
-  hipLaunchKernelGGL((v_finalize_kernel<D>), dim3(B * Hkv), dim3(D), 0, st, (const float*)partial, v_scale,
+  hipLaunchKernelGGL((v_finalize_kernel<D>), dim3(B * Hkv), dim3(1024), 0, st, (const float*)partial, v_scale,
                      v_mean, N, n_chunks, smooth);
   PARO_HIP(hipGetLastError());
   hipLaunchKernelGGL((v_pack_kernel<DT, D>), dim3(nb, Hkv, B), dim3(256), 0, st, vp, v8,
