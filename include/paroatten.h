@@ -177,6 +177,18 @@ int paro_sub_mean(const void* v, int dtype, const void* mean, void* out_f16,
                   int64_t mean_stride_b, int64_t mean_stride_h,
                   int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Block-mask bit packing.  The sparse plan is the one operand of the path that is staged from the
+ * host per layer (paroattention/prefetch_utils.py:34-59 keeps it as torch.bool on the CPU and
+ * paroattention/cogvideox.py:188-213 copies one [H,nb,nb] slice per call); as bits it is 8x smaller
+ * in pinned memory and on the wire.  Bit i of byte j = element 8j+i (numpy.packbits, bitorder
+ * "little").  mask: n bytes of 0/1 (nonzero counts as 1 when packing); bits: paro_mask_bits_bytes(n)
+ * bytes.  Both pointers 16-byte aligned, on the device.
+ * ------------------------------------------------------------------------------------------- */
+int64_t paro_mask_bits_bytes(int64_t n);
+int paro_mask_pack(const uint8_t* mask, uint8_t* bits, int64_t n, void* stream);
+int paro_mask_unpack(const uint8_t* bits, uint8_t* mask, int64_t n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

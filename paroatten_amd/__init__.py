@@ -12,10 +12,14 @@ from . import _lib
 
 _lib.load()  # fail at import time if libparoatten_hip.so is missing: there is no fallback path
 
-from . import _fused, _qattn_sm80, _rope, core, permute, quant  # noqa: E402
+from . import _fused, _qattn_sm80, _rope, cogvideox, core, permute, plans, prefetch_utils, quant, wan  # noqa: E402
+from .cogvideox import PARO_CogVideoXAttnProcessor, PARO_CogVideoXAttnProcessor2_0  # noqa: E402
 from .core import paroattn, paroattn_qk_int8_pv_fp16_cuda  # noqa: E402
+from .wan import PARO_WanAttnProcessor, PARO_WanAttnProcessor2_0, set_paro_processors  # noqa: E402
 
-__all__ = ["paroattn", "paroattn_qk_int8_pv_fp16_cuda", "install_alias"]
+__all__ = ["paroattn", "paroattn_qk_int8_pv_fp16_cuda", "PARO_CogVideoXAttnProcessor2_0",
+           "PARO_CogVideoXAttnProcessor", "PARO_WanAttnProcessor2_0", "PARO_WanAttnProcessor",
+           "set_paro_processors", "install_alias"]
 
 
 def install_alias(name: str = "paroattention"):
@@ -26,4 +30,7 @@ def install_alias(name: str = "paroattention"):
     for sub in list(sys.modules):
         if sub.startswith(__name__ + "."):
             sys.modules[name + sub[len(__name__):]] = sys.modules[sub]
+    # the reference keeps the Wan twin of prefetch_utils in its own module (paroattention/prefetch_wan.py)
+    sys.modules[name + ".prefetch_wan"] = prefetch_utils
+    pkg.prefetch_wan = prefetch_utils
     return pkg

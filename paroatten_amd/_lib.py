@@ -49,6 +49,9 @@ SIGNATURES = {
                                       _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
     "paro_permute_inv": (c_int, [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
     "paro_permute_index_map": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
+    "paro_mask_bits_bytes": (c_int64, [_L]),
+    "paro_mask_pack": (c_int, [_P, _P, _L, _P]),
+    "paro_mask_unpack": (c_int, [_P, _P, _L, _P]),
     "paro_sub_mean": (c_int, [_P, _I, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
 }
 
@@ -63,7 +66,7 @@ def load():
     path = Path(os.environ.get("PAROATTEN_LIB", LIB_PATH))
     if not path.exists():
         raise ImportError(
-            f"{path} is not built: run `python -m paroatten_amd.build` (hipcc, gfx950). "
+            f"{path} is not built: run `python paroatten_amd/build.py` (hipcc, gfx950). "
             "paroatten_amd has no fallback path."
         )
     lib = ctypes.CDLL(str(path))

@@ -1,6 +1,9 @@
 """Build libparoatten_hip.so (device code for gfx950 only) with hipcc, in-tree.
 
-    python -m paroatten_amd.build [--force]
+    python paroatten_amd/build.py
+
+(run as a script, not with -m: importing the package loads the library, which fails while the
+library is missing or older than the header)
 
 No hipify, no torch headers: the library is plain HIP behind a C ABI (include/paroatten.h).
 IEEE fp32 arithmetic is part of the quantisation / RoPE specification, so fast-math stays off and
@@ -18,7 +21,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIBDIR = PKG / "lib"
 LIB = LIBDIR / "libparoatten_hip.so"
-SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "rope_permute.hip", "attn_sparse.hip"]
+SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "rope_permute.hip", "mask_bits.hip", "attn_sparse.hip"]
 ARCH = "gfx950"
 
 FLAGS = [

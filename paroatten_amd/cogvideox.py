@@ -1,0 +1,204 @@
+"""CogVideoX attention processor: the reference's `paroattention.cogvideox`
+(paroattention/cogvideox.py:22-250) on the fused kernels.
+
+`PARO_CogVideoXAttnProcessor2_0` keeps the reference's constructor, injected attributes
+(`permute_plan`, `i_block`, `i_timestep`, and `sparse_mask` or `prefetch_stream`), call signature,
+return value and `get_time_stats()`.  What changes underneath:
+  * RoPE and the per-head permutation of Q, K, V are one launch that reads the projections in
+    their native token-major memory ([B,N,H*D] viewed as [B,H,N,D] through strides): no
+    transpose copy, no in-place rotate pass, no Python loop over heads, no host sync;
+  * V stays bf16/fp16 (the FP8 conversion is inside the attention entry point);
+  * the inverse permutation writes token-major memory directly, so the reshape for the output
+    projection is a view;
+  * (F,H,W), literals in the reference (cogvideox.py:31-33), are the `grid` argument/attribute;
+  * timing is kept by events that are only read in get_time_stats(): no synchronize per call.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from . import _qattn_sm80 as qattn
+from . import permute as PM
+from .permute import permute_attn_out, permute_qk  # noqa: F401  (same module-level names as the reference)
+from .quant import per_warp_int8 as per_warp_int8_cuda
+
+COG_GRID = (13, 30, 45)   # frames x height x width of CogVideoX-5b latents after patching (cogvideox.py:31-33)
+
+
+class _PathTimer:
+    """start/stop event pairs folded into a running total without ever blocking the caller."""
+
+    def __init__(self):
+        self.total_ms = 0.0
+        self._pending = []
+
+    def start(self):
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        self._pending.append((s, e))
+        return e
+
+    def fold(self, block: bool):
+        keep = []
+        for s, e in self._pending:
+            if block:
+                e.synchronize()
+            if e.query():
+                self.total_ms += s.elapsed_time(e)
+            else:
+                keep.append((s, e))
+        self._pending = keep
+
+
+class _ParoProcessorBase:
+    """State and helpers shared by the CogVideoX and Wan processors."""
+
+    def __init__(self, grid: Optional[Sequence[int]] = None, smooth_k: bool = False, exact_exp: bool = False):
+        if not hasattr(F, "scaled_dot_product_attention"):
+            raise ImportError("this attention processor requires PyTorch 2.0 or newer")
+        self.grid = None if grid is None else tuple(int(x) for x in grid)
+        self.smooth_k = smooth_k
+        self.exact_exp = exact_exp
+        self._timer = _PathTimer()
+        self.time_accum = {"total": 0.0}
+        self.call_count = 0
+        self._orders_cache = {}
+        self._table_cache = (None, None, None)
+        self.i_timestep = 0
+        self.i_block = 0
+
+    # ---- plan / mask plumbing ---------------------------------------------------------------
+    def _orders(self, device) -> torch.Tensor:
+        key = (id(self.permute_plan), int(self.i_block), str(device))
+        o = self._orders_cache.get(key)
+        if o is None:
+            o = PM.head_orders(self.permute_plan, int(self.i_block), device)
+            self._orders_cache = {key: o}
+        return o
+
+    def _mask(self) -> torch.Tensor:
+        """bool [H,nb,nb] on the device, shared by the batch (the reference stacks it per CFG
+        branch, cogvideox.py:188-193; the kernel takes a batch stride of 0 instead)."""
+        ps = getattr(self, "prefetch_stream", None)
+        if ps is not None:
+            return ps.mask_for(self.i_timestep, self.i_block)
+        m = self.sparse_mask[self.i_timestep, self.i_block]
+        if m.dtype != torch.bool:
+            m = m.bool()
+        return m
+
+    def _grid_for(self, n_img: int, known) -> Tuple[int, int, int]:
+        g = self.grid
+        if g is None:
+            g = known.get(n_img)
+        if g is None or g[0] * g[1] * g[2] != n_img:
+            raise ValueError(f"{n_img} image tokens do not match grid {g}: set the processor's `grid` to (F, H, W)")
+        return g
+
+    @staticmethod
+    def _rope_permute(query, key, value, orders, grid, n_text, cos, sin, rotate_key=True):
+        """One launch when q, k, v share strides (plain projections); otherwise (a norm layer returned
+        q/k in another memory order than v, or keys that must not be rotated) one launch per group."""
+        same = query.stride() == key.stride() == value.stride()
+        if same and (rotate_key or cos is None):
+            return PM.rope_permute(query, key, value, orders, grid, n_text, cos, sin)
+        if rotate_key and query.stride() == key.stride():
+            qp, kp, _ = PM.rope_permute(query, key, None, orders, grid, n_text, cos, sin)
+        else:
+            qp, _, _ = PM.rope_permute(query, None, None, orders, grid, n_text, cos, sin)
+            _, kp, _ = PM.rope_permute(None, key, None, orders, grid, n_text,
+                                       cos if rotate_key else None, sin if rotate_key else None)
+        _, _, vp = PM.rope_permute(None, None, value, orders, grid, n_text)
+        return qp, kp, vp
+
+    def _sparse_attention(self, qp, kp, vp, sm_scale):
+        km = kp.mean(dim=2, keepdim=True) if self.smooth_k else None
+        q8, qs, k8, ks = per_warp_int8_cuda(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64, tensor_layout="HND")
+        out = torch.empty_like(qp)
+        qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, vp, out, qs, ks, 1, 0, 2, sm_scale, 0, self._mask(),
+                                            exact_exp=self.exact_exp)
+        return out
+
+    def get_time_stats(self):
+        self._timer.fold(block=True)
+        self.time_accum["total"] = self._timer.total_ms
+        return {"total_ms": self.time_accum["total"]}
+
+
+class PARO_CogVideoXAttnProcessor2_0(_ParoProcessorBase):
+    r"""Joint text+video self-attention of CogVideoX with PAROAttention in place of dense SDPA
+    (paroattention/cogvideox.py:112-250).  `i_timestep < 0` selects dense SDPA, as there (:215-221)."""
+
+    def _tables(self, image_rotary_emb, device):
+        cos, sin = image_rotary_emb
+        key = (cos.data_ptr(), sin.data_ptr(), str(device))
+        if self._table_cache[0] != key:
+            self._table_cache = (key, cos.to(device=device, dtype=torch.float32).contiguous(),
+                                 sin.to(device=device, dtype=torch.float32).contiguous())
+        return self._table_cache[1], self._table_cache[2]
+
+    def __call__(self, attn, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,
+                 attention_mask: Optional[torch.Tensor] = None,
+                 image_rotary_emb: Optional[torch.Tensor] = None):
+        text_seq_length = encoder_hidden_states.size(1)
+        hidden_states = torch.cat([encoder_hidden_states, hidden_states], dim=1)
+        batch_size, sequence_length, _ = hidden_states.shape
+
+        query = attn.to_q(hidden_states)
+        key = attn.to_k(hidden_states)
+        value = attn.to_v(hidden_states)
+        head_dim = key.shape[-1] // attn.heads
+        # [B,H,N,D] views of the token-major projections: the permutation kernel follows the strides
+        query = query.view(batch_size, -1, attn.heads, head_dim).transpose(1, 2)
+        key = key.view(batch_size, -1, attn.heads, head_dim).transpose(1, 2)
+        value = value.view(batch_size, -1, attn.heads, head_dim).transpose(1, 2)
+        if attn.norm_q is not None:
+            query = attn.norm_q(query)
+        if attn.norm_k is not None:
+            key = attn.norm_k(key)
+
+        grid = self._grid_for(sequence_length - text_seq_length, {COG_GRID[0] * COG_GRID[1] * COG_GRID[2]: COG_GRID})
+        cos = sin = None
+        if image_rotary_emb is not None:
+            cos, sin = self._tables(image_rotary_emb, query.device)
+        dense = self.i_timestep < 0
+        if dense:
+            orders = torch.zeros(attn.heads, dtype=torch.int32, device=query.device)   # order 0 = identity
+        else:
+            orders = self._orders(query.device)
+        # keys of a cross-attention layer are not rotated (cogvideox.py:170-172)
+        qp, kp, vp = self._rope_permute(query, key, value, orders, grid, text_seq_length, cos, sin,
+                                        rotate_key=not getattr(attn, "is_cross_attention", False))
+
+        done = self._timer.start()
+        token_major = torch.empty((batch_size, sequence_length, attn.heads, head_dim), dtype=query.dtype,
+                                  device=query.device)
+        if dense:
+            if attention_mask is not None:
+                attention_mask = attn.prepare_attention_mask(attention_mask, sequence_length, batch_size)
+                attention_mask = attention_mask.view(batch_size, attn.heads, -1, attention_mask.shape[-1])
+            out = F.scaled_dot_product_attention(qp, kp, vp, attn_mask=attention_mask, dropout_p=0.0, is_causal=False)
+            token_major.copy_(out.transpose(1, 2))
+            done.record()
+        else:
+            out = self._sparse_attention(qp, kp, vp, 1.0 / (head_dim ** 0.5))
+            done.record()
+            PM.permute_inverse(out, orders, grid, text_seq_length, out=token_major.transpose(1, 2))
+        self.call_count += 1
+        if len(self._timer._pending) >= 64:
+            self._timer.fold(block=False)
+
+        hidden_states = token_major.view(batch_size, sequence_length, attn.heads * head_dim)
+        hidden_states = attn.to_out[0](hidden_states)   # linear projection
+        hidden_states = attn.to_out[1](hidden_states)   # dropout
+        encoder_hidden_states, hidden_states = hidden_states.split(
+            [text_seq_length, hidden_states.size(1) - text_seq_length], dim=1)
+        return hidden_states, encoder_hidden_states
+
+
+# the same class under its name without the diffusers version suffix
+PARO_CogVideoXAttnProcessor = PARO_CogVideoXAttnProcessor2_0

@@ -75,13 +75,22 @@ def rope_permute(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Option
     return tuple(outs)
 
 
-def permute_inverse(o: torch.Tensor, orders: torch.Tensor, grid: Sequence[int], n_text: int) -> torch.Tensor:
-    """out[b,h,t] = o[b,h,perm_h(t)]: undoes rope_permute's token order on the attention output."""
+def permute_inverse(o: torch.Tensor, orders: torch.Tensor, grid: Sequence[int], n_text: int,
+                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[b,h,t] = o[b,h,perm_h(t)]: undoes rope_permute's token order on the attention output.
+    `out`, if given, is any [B,H,N,D] view with a contiguous last dimension that does not overlap `o`
+    (e.g. the transpose of an [B,N,H,D] buffer, which makes the result token-major for the output
+    projection without another pass)."""
     _check_hnd(o, "attn_out")
     B, H, N, D = o.shape
     _check_orders(orders, H)
     F, Hh, W = (int(x) for x in grid)
-    out = torch.empty((B, H, N, D), dtype=o.dtype, device=o.device)
+    if out is None:
+        out = torch.empty((B, H, N, D), dtype=o.dtype, device=o.device)
+    else:
+        _check_hnd(out, "out")
+        if out.shape != o.shape or out.dtype != o.dtype or out.device != o.device:
+            raise RuntimeError("out must have attn_out's shape, dtype and device")
     check(load().paro_permute_inv(ptr(o), ptr(out), _lib.DTYPE_CODE[o.dtype], ptr(orders), B, H, N, D, int(n_text),
                                   F, Hh, W, o.stride(0), o.stride(1), o.stride(2),
                                   out.stride(0), out.stride(1), out.stride(2), stream_of(o)))

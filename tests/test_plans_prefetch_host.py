@@ -1,0 +1,83 @@
+"""Host-side logic around the path (no GPU): plan file formats, mask expansion for the kernel, the
+timestep callback's arithmetic, bit packing of masks."""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from paroatten_amd import plans, prefetch_utils
+
+
+def test_plan_files_round_trip(tmp_path):
+    p_path, s_path = plans.write_synthetic_plans(tmp_path, T=2, L=3, H=4, nb_img=10, density=0.4, seed=3)
+    pp = plans.load_permute_plan(p_path)
+    sp = plans.load_sparse_plan(s_path)
+    assert pp["permute"].shape == (3, 4) and pp["permute"].dtype == torch.int64
+    assert int(pp["permute"].min()) >= 0 and int(pp["permute"].max()) <= 5
+    assert pp["empty"].shape == (3, 4) and pp["empty"].dtype == torch.bool
+    assert sp["sparse"].shape == (2, 3, 4, 10, 10) and sp["sparse"].dtype == torch.bool
+    # exact block count per head, diagonal kept
+    assert torch.all(sp["sparse"].sum(dim=(-1, -2)) == max(40, int((torch.arange(10)[:, None] - torch.arange(10)).abs().le(2).sum())))
+    assert torch.all(torch.diagonal(sp["sparse"], dim1=-2, dim2=-1))
+    assert torch.allclose(sp["dense_rate"], sp["sparse"].float().mean(dim=(-1, -2)))
+
+
+def test_plan_validation():
+    with pytest.raises(ValueError):
+        plans.check_permute_plan({"permute": torch.tensor([[0, 6]])})
+    with pytest.raises(ValueError):
+        plans.check_permute_plan({"perm": torch.zeros(1, 1)})
+    ok = plans.check_permute_plan({"permute": torch.tensor([[0, 5]], dtype=torch.int32)})
+    assert ok["empty"].shape == (1, 2) and not ok["empty"].any()
+
+
+def test_cog_kernel_mask_text_blocks():
+    """pipeline_cogvideox.py:80,99-100: 4 leading rows/columns of ones, last row/column True;
+    the image part is untouched elsewhere."""
+    g = torch.Generator().manual_seed(0)
+    s = torch.rand(2, 1, 3, 274, 274, generator=g) < 0.2
+    m = plans.cog_kernel_mask(s)
+    assert m.shape == (2, 1, 3, 278, 278)
+    assert m[..., :4, :].all() and m[..., :, :4].all()
+    assert m[..., -1, :].all() and m[..., :, -1].all()
+    assert torch.equal(m[..., 4:-1, 4:-1], s[..., :-1, :-1])
+    w = plans.wan_kernel_mask(s)
+    assert w.shape == s.shape and w[..., -1, :].all() and w[..., :, -1].all()
+    assert torch.equal(w[..., :-1, :-1], s[..., :-1, :-1])
+    assert not s[..., -1, :].all()   # the input was not modified
+
+
+@pytest.mark.parametrize("step,total,T,expect", [
+    (0, 50, 10, 0), (3, 50, 10, 0), (4, 50, 10, 1), (48, 50, 10, 9), (49, 50, 10, 10),
+    (50, 50, 10, 0), (0, 4, 4, 1), (2, 4, 4, 3), (7, 8, 4, 4),
+])
+def test_mask_timestep_index(step, total, T, expect):
+    """prefetch_utils.py:22-25, worked by hand: int(((step % total)+1)/total*T)."""
+    assert prefetch_utils.mask_timestep_index(step, total, T) == expect
+
+
+@pytest.mark.parametrize("blocks_attr", ["transformer_blocks", "blocks"])
+def test_timestep_callback_writes_every_processor(blocks_attr):
+    procs = [types.SimpleNamespace(i_timestep=-5) for _ in range(3)]
+    blocks = [types.SimpleNamespace(attn1=types.SimpleNamespace(processor=p)) for p in procs]
+    transformer = types.SimpleNamespace(**{blocks_attr: blocks})
+    pipe = types.SimpleNamespace(transformer=transformer, scheduler=types.SimpleNamespace(timesteps=list(range(20))))
+    cb = prefetch_utils.TimestepCallback(num_timestep_for_sparse_mask=10)
+    kw = {"latents": None}
+    assert cb.on_step_end(pipe, 5, torch.tensor(801.0), kw) is kw
+    assert transformer.i_timestep == 3 and all(p.i_timestep == 3 for p in procs)
+    assert cb.timestep_history[0]["step"] == 5 and cb.timestep_history[0]["timestep"] == 801.0
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 127, 128, 1000])
+def test_pack_mask_bits_matches_numpy(n):
+    g = torch.Generator().manual_seed(n)
+    m = torch.rand(3, n, generator=g) < 0.5
+    bits = prefetch_utils.pack_mask_bits(m)
+    assert bits.shape[1] % 16 == 0 and bits.shape[1] >= (n + 7) // 8
+    back = np.unpackbits(bits.numpy(), axis=1, bitorder="little")[:, :n]
+    assert np.array_equal(back.astype(bool), m.numpy())
+    # element 8j+i is bit i of byte j
+    j, i = (n - 1) // 8, (n - 1) % 8
+    assert bool((int(bits[0, j]) >> i) & 1) == bool(m[0, n - 1])
