@@ -127,8 +127,11 @@ __device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, u
                                            soffset, 0, 0);
 }
 
+// Waves per SIMD the register budget is set for: the D = 64 production variants fit 168 registers.
+#define PARO_ATTN_WAVES_PER_SIMD ((D == 64 && !CAUSAL && !DUMP && !LSE) ? 3 : 2)
+
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
-__global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p) {
+__global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_kernel(const AttnParams p) {
   using Lds = AttnLds<D>;
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
   constexpr int DT_TILES = D / 32;  // 32-channel tiles of O^T
@@ -255,9 +258,12 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
       const int row = 32 * mt + l32;
       kr_off[ks * 2 + mt] = row * D + (((2 * ks + lh) ^ Lds::swz(row)) * 16);
     }
+  auto read_k_frag = [&](int ST, int i) {
+    kfrag[i] = *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + kr_off[i]);
+  };
   auto read_k_frags = [&](int ST) {
 #pragma unroll
-    for (int i = 0; i < 2 * KS; i++) kfrag[i] = *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + kr_off[i]);
+    for (int i = 0; i < 2 * KS; i++) read_k_frag(ST, i);
   };
   // S^T tile: 64 kv-rows (2 MFMA row tiles) x 32 q-columns.  The accumulators start at the bit
   // pattern of 1.5*2^23: the int32 result then READS as the float 12582912 + S exactly
@@ -297,11 +303,15 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
     for (int i = 0; i < 16; i++) o_acc[dt][i] = 0.f;
-  // every row of this 32x32 tile ends up holding the row sums of P~ (only element 0 is read)
-  v16f d_acc;
-#pragma unroll
-  for (int i = 0; i < 16; i++) d_acc[i] = 0.f;
-  v8i ones = {FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES, FP8_ONES};
+  // Row sums of the ROUNDED P~ from the matrix pipe, on the cheapest shape that fits: in a
+  // 16x16x128 product the B lanes 16g..16g+15 (g = lane/16) supply k-range 32g..32g+31 of columns
+  // 0..15, and P~'s fragment has q-row lane%32 and kv-half lane/32 there, i.e. k-ranges 0 and 2 are
+  // the two kv-halves of q-rows 0..15 and k-ranges 1 and 3 those of q-rows 16..31.  With A row 0 =
+  // ones on k-ranges {0,2} and A row 1 = ones on {1,3} (A lane: row lane%16, k-range lane/16), lanes
+  // 0..15 get d_acc[0] = row sum of q-row lane and d_acc[1] = that of q-row lane+16.
+  v4f d_acc = {0.f, 0.f, 0.f, 0.f};
+  const int sel_word = ((lane & 15) == ((lane >> 4) & 1)) ? FP8_ONES : 0;
+  v8i ones = {sel_word, sel_word, sel_word, sel_word, sel_word, sel_word, sel_word, sel_word};
   asm volatile("" : "+v"(ones));  // same: resident constant operand
   float m_i = -1e30f;
   float d_exact = 0.f;  // LSE only: sum of the unrounded P~ of this lane's 32 kv-columns per block
@@ -339,7 +349,7 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
                      vfrag[idx][1][0], vfrag[idx][1][1], vfrag[idx][1][2], vfrag[idx][1][3]};
       o_acc[idx] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, pf, o_acc[idx], 0, 0, 0, 0, 0, 0);
     } else {
-      d_acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
+      d_acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
     }
   };
   auto read_v_frags = [&](int ST) {
@@ -361,7 +371,6 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     load_k(kb_3, sk0);
     load_v(kb_1, sv1);
     const int kidx_v = (int)klist[it + 4];
-    read_k_frags(sk1);
     read_v_frags(svp);
     const float c_next = qsc * clist[it + 1];
 
@@ -424,19 +433,26 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     const float bias8 = fmaf(-S_MAGIC_F, c8, 8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT);
     // MFMA issue plan: the pending P.V first (its operands are ready), S^T row tile 0 of the next
     // block once chunk 3 has read the last of the current one, row tile 1 after chunk 7
+    // The K fragments of the next block (k-step r, both row tiles) are fetched from LDS right after
+    // the P.V MFMA that was the last reader of V fragment r: the two fragment sets never live at the
+    // same time and share registers.
     auto mfma_after_chunk = [&](int r) {
+      if (r < DT_TILES) {
+        pv_one(pf_p, r);
+        read_k_frag(sk1, 2 * r);
+        read_k_frag(sk1, 2 * r + 1);
+      }
       if constexpr (D == 64) {
-        if (r < 3) pv_one(pf_p, r);
+        if (r == 2) pv_one(pf_p, 2);
         else if (r == 3) qk_one(0);
         else if (r == 4) qk_one(1);
         else if (r == 7) { qk_one(2); qk_one(3); }
       } else {
-        if (r < 3) pv_one(pf_p, r);
-        else if (r == 3) { pv_one(pf_p, 3); pv_one(pf_p, 4); qk_one(0); }
-        else if (r == 4) qk_one(1);
+        if (r == 3) pv_one(pf_p, 4);
+        else if (r == 4) { qk_one(0); qk_one(1); }
         else if (r == 5) qk_one(2);
         else if (r == 6) qk_one(3);
-        else { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
+        else if (r == 7) { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
       }
     };
     // Fast path: the e4m3 byte of 2^t is built directly: byte = rne(8*(t + 7) + FAST_EXP_SHIFT), i.e.
@@ -495,7 +511,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
     if constexpr (LSE) d_exact += rs;
     if (it + 1 < cnt) dump_s(kb_1);
     if (refresh) {
-      d_acc[0] *= alpha;
+      d_acc[0] *= alpha;                                          // lanes 0..15: q-row lane
+      d_acc[1] *= __shfl(alpha, (lane & 15) + 16, 64);            // and q-row lane+16
 #pragma unroll
       for (int dt = 0; dt < DT_TILES; dt++)
 #pragma unroll
@@ -532,7 +549,8 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_kernel(const AttnParams p)
   }
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------
-  const float d_tot = d_acc[0];
+  const float d_lo = __shfl(d_acc[0], l32 & 15, 64), d_hi = __shfl(d_acc[1], l32 & 15, 64);
+  const float d_tot = l32 < 16 ? d_lo : d_hi;
   const float inv = 1.0f / d_tot;
   if (qrow < p.Nq) {
     const float* vsc = p.v_scale + bhk * D;
