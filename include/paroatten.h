@@ -168,6 +168,39 @@ int paro_permute_inv(const void* in, void* out, int dtype, const int32_t* orders
 int paro_permute_index_map(int32_t* idx, const int32_t* orders, int H, int F, int Hh, int W, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * (3b) The whole preparation of the attention operands in one pass: RoPE + permutation + INT8
+ * quantisation of Q and K + FP8 packing of the permuted V.  Same results as the chain
+ * paro_rope_permute_fwd -> paro_quant_int8 (Q: groups of 32 tokens, K: groups of 64, optional
+ * mean) -> paro_v_fp8_pack (INT8 tensors and scales bit-identical; V's mean is summed in source
+ * order, so it may differ in the last fp32 bit), i.e. as what the processors do between the projections and the
+ * attention call (paroattention/cogvideox.py:167-186 with quant.py:105-180 and, for V,
+ * quant.py:224-293), without writing the permuted 16-bit tensors.
+ * q, k, v: [B,H,N,D] through the three input strides (shared by the three tensors).  k_mean: NULL
+ * or [B,H,D] in the input dtype through mean strides (subtracted from the rotated K before
+ * quantisation).  Outputs, all contiguous: q8, k8 int8 [B,H,N,D]; q_scale f32 [B,H,2*ceil(N/64)];
+ * k_scale f32 [B,H,ceil(N/64)]; v8 paro_v_fp8_bytes(); v_scale, v_mean f32 [B,H,D].
+ * workspace: paro_prep_workspace_bytes() bytes.
+ * paro_rope_k_mean: k_mean[b,h,:] = mean over tokens of the ROTATED K, rounded to the input dtype
+ * (what `km = k.mean(dim=seq)` gives the reference's quantiser after the processor's RoPE).
+ * ------------------------------------------------------------------------------------------- */
+int64_t paro_prep_workspace_bytes(int B, int H, int N, int D);
+int paro_rope_permute_quant_fwd(const void* q, const void* k, const void* v, int dtype,
+                                const float* cos, const float* sin, const int32_t* orders,
+                                const void* k_mean,
+                                int8_t* q8, float* q_scale, int8_t* k8, float* k_scale,
+                                uint8_t* v8, float* v_scale, float* v_mean,
+                                void* workspace, int64_t workspace_bytes,
+                                int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                                int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_n,
+                                int64_t mean_stride_b, int64_t mean_stride_h,
+                                int smooth_v, void* stream);
+int paro_rope_k_mean(const void* k, int dtype, const float* cos, const float* sin, void* k_mean,
+                     void* workspace, int64_t workspace_bytes,
+                     int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                     int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                     int64_t mean_stride_b, int64_t mean_stride_h, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * V helpers kept for API completeness of paroattention._fused (csrc/fused/fused.cu:200-260,
  * 770-848): out_f16[b,h,n,:] = fp16(v - mean[b,h,:]) (bf16 input: subtract in bf16 first).
  * ------------------------------------------------------------------------------------------- */

@@ -326,7 +326,7 @@ def rope_table_cog(head_dim: int, grid: Sequence[int], theta: float = 10000.0):
 # ----------------------------------------------------------------------------------------
 def per_channel_fp8(v: torch.Tensor, scale_max: float = 448.0, smooth_v: bool = True):
     """Per-(b,h,channel) e4m3 quantisation of V [B,H,N,D]: vm = mean over the N tokens,
-    scale = max|v - vm| / scale_max, v8 = e4m3_rne_satfinite((v - vm)/scale).  Returned in
+    scale = max|v - vm| / scale_max, v8 = e4m3_rne_satfinite((v - vm) * (scale_max / max|v - vm|)).  Returned in
     token-major form [B,H,N,D] (the reference's transposed+shuffled storage,
     fused.cu:262-313, is an NVIDIA fragment layout and not part of the arithmetic).
     Deviation kept on purpose: the mean divides by N, not by ceil16(N) (fused.cu:335,381)."""
@@ -338,7 +338,9 @@ def per_channel_fp8(v: torch.Tensor, scale_max: float = 448.0, smooth_v: bool = 
         vm = None
     amax = vf.abs().amax(dim=2)
     scale = amax / scale_max
-    v8 = (vf / scale.clamp_min(1e-30).unsqueeze(2)).clamp(-scale_max, scale_max).to(torch.float8_e4m3fn)
+    # fused.cu:399,414: multiply by recp_scale = scale_max / amax (a constant channel gives 0, not NaN)
+    recp = torch.where(amax > 0, scale_max / amax, torch.zeros_like(amax))
+    v8 = (vf * recp.unsqueeze(2)).clamp(-scale_max, scale_max).to(torch.float8_e4m3fn)
     return v8, scale, vm
 
 

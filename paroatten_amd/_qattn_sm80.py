@@ -120,6 +120,49 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
     return lse
 
 
+def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_scale, sm_scale, sparse,
+                          is_causal=0, return_lse=0, exact_exp=False):
+    """The attention kernel alone, on operands that are already in its formats (HND, contiguous):
+    q8/k8 int8 [B,H,N,D] / [B,Hkv,Nk,D], v8 = FP8 tiles from paro_v_fp8_pack or the fused
+    preparation, v_scale / v_mean f32 [B,Hkv,D] (v_mean None: V was not mean-smoothed).  No
+    counterpart in the reference, whose extension converts V on every call."""
+    for t, n in ((q8, "query"), (k8, "key"), (v8, "value"), (output, "output"), (query_scale, "query_scale"),
+                 (key_scale, "key_scale"), (v_scale, "v_scale"), (sparse, "sparse")):
+        _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
+        _chk(t.is_contiguous() or n == "output", f"Tensor {n} must be contiguous")
+    _chk(q8.dtype == torch.int8 and k8.dtype == torch.int8, "Tensor query/key must have dtype (torch::kInt8)")
+    _chk(q8.dim() == 4 and k8.dim() == 4, "Tensor query/key must have dimension number (4)")
+    B, H, Nq, D = q8.shape
+    Hkv, Nk = k8.size(1), k8.size(2)
+    if D not in (64, 128):
+        raise ValueError(f"Unsupported head dim: {D}")
+    if H % Hkv != 0:
+        raise ValueError(f"num_qo_heads ({H}) must be divisible by num_kv_heads ({Hkv})")
+    nbq, nbk = (Nq + 63) // 64, (Nk + 63) // 64
+    _chk(v8.numel() * v8.element_size() == load().paro_v_fp8_bytes(B, Hkv, Nk, D), "Tensor value has the wrong size for FP8 tiles")
+    _chk(tuple(query_scale.shape) == (B, H, nbq * 2) and tuple(key_scale.shape) == (B, Hkv, nbk),
+         "Tensor query_scale / key_scale must have shapes (B, H, 2*nbq) / (B, Hkv, nbk)")
+    _chk(tuple(v_scale.shape) == (B, Hkv, D) and (v_mean is None or tuple(v_mean.shape) == (B, Hkv, D)),
+         "Tensor v_scale / v_mean must have shape (B, Hkv, head_dim)")
+    _chk(tuple(output.shape) == (B, H, Nq, D) and output.stride(-1) == 1 and output.dtype in _lib.DTYPE_CODE,
+         "Tensor output must be float16/bfloat16 [B,H,N,D] with a contiguous last dimension")
+    _chk(sparse.dtype in (torch.bool, torch.uint8), "Tensor sparse must have dtype (torch::kBool)")
+    if sparse.dim() == 4:
+        _chk(tuple(sparse.shape) == (B, H, nbq, nbk), f"Tensor sparse must have shape ({B}, {H}, {nbq}, {nbk})")
+        sparse_bs = sparse.stride(0)
+    else:
+        _chk(tuple(sparse.shape) == (H, nbq, nbk), f"Tensor sparse must have shape ([{B},] {H}, {nbq}, {nbk})")
+        sparse_bs = 0
+    lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q8.device) if return_lse else torch.empty(0)
+    check(load().paro_attn_sparse_fwd(
+        ptr(q8), ptr(k8), ptr(v8), ptr(query_scale), ptr(key_scale), ptr(v_scale), ptr(v_mean), ptr(sparse), sparse_bs,
+        ptr(output), _lib.DTYPE_CODE[output.dtype], ptr(lse) if return_lse else None, None,
+        B, H, Hkv, Nq, Nk, D, q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
+        output.stride(0), output.stride(1), output.stride(2), float(sm_scale), int(is_causal),
+        _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0, stream_of(q8)))
+    return lse
+
+
 def _prototype(name):
     def fn(*args, **kwargs):
         raise NotImplementedError(

@@ -77,12 +77,17 @@ __device__ __forceinline__ void cvt_pk_fp8(int& w, float a, float b) {
   else asm("v_cvt_pk_fp8_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));  // upper half: don't care, overwritten next
 }
 
-// float -> unsigned byte (round to nearest even, clamped to [0,255]) into byte BYTE of w; FIRST starts
-// a fresh word (whatever the other bytes hold is overwritten by the three calls that follow)
-template <int BYTE, bool FIRST>
-__device__ __forceinline__ void cvt_pk_u8(int& w, float a) {
-  if constexpr (FIRST) asm("v_cvt_pk_u8_f32 %0, %1, %2, %0" : "=v"(w) : "v"(a), "n"(BYTE));
-  else asm("v_cvt_pk_u8_f32 %0, %1, %2, %0" : "+v"(w) : "v"(a), "n"(BYTE));
+// two floats in [0,1] -> round(x * 65535) as two unsigned 16-bit fields (negative inputs give 0)
+__device__ __forceinline__ int cvt_pknorm_u16(float a, float b) {
+  int w;
+  asm("v_cvt_pknorm_u16_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));
+  return w;
+}
+
+__device__ __forceinline__ int lshl8_or(int hi, int lo) {
+  int w;
+  asm("v_lshl_or_b32 %0, %1, 8, %2" : "=v"(w) : "v"(hi), "v"(lo));
+  return w;
 }
 
 __device__ __forceinline__ float partner_max(float x) {
@@ -429,8 +434,8 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     //    pending P.V of the PREVIOUS block.  All their operands are ready before the stream starts.
     float rs = 0.f;
     const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
-    const float c8 = 8.0f * c;
-    const float bias8 = fmaf(-S_MAGIC_F, c8, 8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT);
+    const float c8 = (8.0f / 65535.0f) * c;
+    const float bias8 = fmaf(-S_MAGIC_F, c8, (8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT) * (1.0f / 65535.0f));
     // MFMA issue plan: the pending P.V first (its operands are ready), S^T row tile 0 of the next
     // block once chunk 3 has read the last of the current one, row tile 1 after chunk 7
     // The K fragments of the next block (k-step r, both row tiles) are fetched from LDS right after
@@ -455,18 +460,18 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
         else if (r == 7) { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
       }
     };
-    // Fast path: the e4m3 byte of 2^t is built directly: byte = rne(8*(t + 7) + FAST_EXP_SHIFT), i.e.
+    // Fast path: the e4m3 byte of 2^t is built directly: byte = round(8*(t + 7) + FAST_EXP_SHIFT), i.e.
     // exponent field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of
-    // two (at most 6 % off, shifted to be centred).  One fma and one byte conversion per element
-    // instead of fma + v_exp_f32 + half a packed FP8 conversion; v_cvt_pk_u8_f32 rounds to nearest
-    // even and clamps to [0, 255], which sends masked (-inf) and underflowing elements to 0.  Its
-    // chunk r = (row tile r/4, byte r%4 of that tile's four words): the four conversions of a chunk
-    // are independent of each other.
-    int wf[8];
+    // two (at most 6 % off, shifted to be centred).  Per word of four weights: four fmas (the affine
+    // map pre-divided by 65535), two v_cvt_pknorm_u16_f32 (each rounds two values to 16-bit integer
+    // fields, clamping negatives, i.e. masked and underflowing elements, to 0) and one shift-or that
+    // interleaves the two pairs into bytes; the lazy maximum keeps every value <= 126, so no field
+    // spills into its neighbour.  Instead of fma + v_exp_f32 + half a packed FP8 conversion per weight.
+    // Chunk r = word r%4 of row tile r/4.
     float u_cur[4], u_nxt[4];
     if constexpr (!EXACT) {
 #pragma unroll
-      for (int q = 0; q < 4; q++) u_cur[q] = fmaf(s[0][4 * q], c8, bias8);
+      for (int q = 0; q < 4; q++) u_cur[q] = fmaf(s[0][q], c8, bias8);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
@@ -476,17 +481,14 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
       if constexpr (!EXACT) {
         // the fmas of the next chunk are issued between this chunk's conversions: every conversion
         // finds its input ready
-        const int byte = r & 3;
-        const int rn = r + 1, mtn = rn >> 2, byten = rn & 3;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          if (rn < 8) u_nxt[q] = fmaf(s[mtn][4 * q + byten], c8, bias8);
-          if (byte == 0) cvt_pk_u8<0, true>(wf[mt * 4 + q], u_cur[q]);
-          else if (byte == 1) cvt_pk_u8<1, false>(wf[mt * 4 + q], u_cur[q]);
-          else if (byte == 2) cvt_pk_u8<2, false>(wf[mt * 4 + q], u_cur[q]);
-          else cvt_pk_u8<3, false>(wf[mt * 4 + q], u_cur[q]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
+        const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
+        if (rn < 8) { u_nxt[0] = fmaf(s[mtn][in0 + 0], c8, bias8); u_nxt[2] = fmaf(s[mtn][in0 + 2], c8, bias8); }
+        const int lo = cvt_pknorm_u16(u_cur[0], u_cur[2]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (rn < 8) { u_nxt[1] = fmaf(s[mtn][in0 + 1], c8, bias8); u_nxt[3] = fmaf(s[mtn][in0 + 3], c8, bias8); }
+        const int hi = cvt_pknorm_u16(u_cur[1], u_cur[3]);
+        __builtin_amdgcn_sched_barrier(0);
+        w = lshl8_or(hi, lo);
 #pragma unroll
         for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
       } else {
@@ -499,14 +501,10 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
         cvt_pk_fp8<false>(w, p0, p1);
         cvt_pk_fp8<true>(w, p2, p3);
       }
-      if constexpr (EXACT) pf[r] = w;
+      pf[r] = w;
       __builtin_amdgcn_sched_barrier(0);
       mfma_after_chunk(r);
       __builtin_amdgcn_sched_barrier(0);
-    }
-    if constexpr (!EXACT) {
-#pragma unroll
-      for (int r = 0; r < 8; r++) pf[r] = wf[r];
     }
     if constexpr (LSE) d_exact += rs;
     if (it + 1 < cnt) dump_s(kb_1);

@@ -1,0 +1,115 @@
+// Device helpers shared by the permutation kernels and the V -> FP8 kernels (gfx950 only).
+#pragma once
+#include "paro_common.hpp"
+
+namespace paro {
+
+constexpr int V_CHUNK = 256;  // tokens per chunk of the per-channel V statistics
+
+// strides of the (f,h,w) coordinates in the permuted order `order`
+__device__ __forceinline__ void order_strides(int order, int F, int Hh, int W, int& sf, int& sh, int& sw) {
+  switch (order) {
+    default:
+    case 0: sf = Hh * W; sh = W;     sw = 1;      break;  // FHW
+    case 1: sf = W * Hh; sw = Hh;    sh = 1;      break;  // FWH
+    case 2: sh = W * F;  sw = F;     sf = 1;      break;  // HWF
+    case 3: sh = F * W;  sf = W;     sw = 1;      break;  // HFW
+    case 4: sw = Hh * F; sh = F;     sf = 1;      break;  // WHF
+    case 5: sw = F * Hh; sf = Hh;    sh = 1;      break;  // WFH
+  }
+}
+
+// two floats -> two 16-bit values (round to nearest even), `lo` in bits 0..15: one instruction on gfx950
+template <int DT>
+__device__ __forceinline__ unsigned pack2_from_f32(float lo, float hi) {
+  unsigned w;
+  if constexpr (DT == PARO_DTYPE_F16) asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(w) : "v"(lo), "v"(hi));
+  else asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(lo), "v"(hi));
+  return w;
+}
+template <int DT>
+__device__ __forceinline__ float lo16_to_f32(unsigned w) {
+  if constexpr (DT == PARO_DTYPE_BF16) return __uint_as_float(w << 16);
+  else return F16x<DT>::to_f32((unsigned short)(w & 0xffffu));
+}
+template <int DT>
+__device__ __forceinline__ float hi16_to_f32(unsigned w) {
+  if constexpr (DT == PARO_DTYPE_BF16) return __uint_as_float(w & 0xffff0000u);
+  else return F16x<DT>::to_f32((unsigned short)(w >> 16));
+}
+// element j (0..7) of a 16-byte piece
+template <int DT>
+__device__ __forceinline__ float elem16_to_f32(const v4i& raw, int j) {
+  const unsigned w = (unsigned)raw[j >> 1];
+  return (j & 1) ? hi16_to_f32<DT>(w) : lo16_to_f32<DT>(w);
+}
+
+// rotation of 8 consecutive channels (4 pairs) of one token; cs/sn: that token's table entries
+template <int DT>
+__device__ __forceinline__ v4i rotate8(const v4i raw, const float* cs, const float* sn) {
+  v4i o;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const float x0 = lo16_to_f32<DT>((unsigned)raw[j]);
+    const float x1 = hi16_to_f32<DT>((unsigned)raw[j]);
+    const float o0 = __fsub_rn(__fmul_rn(x0, cs[2 * j]), __fmul_rn(x1, sn[2 * j]));
+    const float o1 = __fadd_rn(__fmul_rn(x1, cs[2 * j + 1]), __fmul_rn(x0, sn[2 * j + 1]));
+    o[j] = (int)pack2_from_f32<DT>(o0, o1);
+  }
+  return o;
+}
+
+// four values y (|y| <= 127.5, not yet rounded) -> four int8 = rint(y) packed in a word.  Adding
+// 1.5*2^23 rounds to the nearest integer, ties to even, exactly as rintf does (the sum lies in
+// [2^23, 2^24), where floats are the integers), and leaves the two's-complement byte in bits 0..7.
+__device__ __forceinline__ unsigned pack4_rint_i8(float y0, float y1, float y2, float y3) {
+  constexpr float M = 12582912.0f;
+  const unsigned a0 = __float_as_uint(__fadd_rn(y0, M)), a1 = __float_as_uint(__fadd_rn(y1, M));
+  const unsigned a2 = __float_as_uint(__fadd_rn(y2, M)), a3 = __float_as_uint(__fadd_rn(y3, M));
+  const unsigned lo = __builtin_amdgcn_perm(a1, a0, 0x0c0c0400u);  // [a0.b0, a1.b0, 0, 0]
+  const unsigned hi = __builtin_amdgcn_perm(a3, a2, 0x0c0c0400u);
+  return lo | (hi << 16);
+}
+
+// One 64-token V tile held in LDS as 16-bit rows (row pitch PITCH elements) -> (v - mean) * recp as
+// e4m3 in the fragment order of the P.V MFMA: 16-byte piece c = (dt, mt, lane) holds channel
+// 32*dt + lane%32 of tokens 32*mt + 8*g + 4*(lane/32) + q, byte 4*g + q.  recp = 448 / max|v - mean|
+// (0 for a constant channel), as MeanScaleKernel of the reference forms it
+// (csrc/fused/fused.cu:399,414).  256 threads.
+template <int DT, int D, int PITCH>
+__device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t* ob, const float* v_recp,
+                                            const float* v_mean, int tok0, int N, int t) {
+#pragma unroll
+  for (int c = t; c < 4 * D; c += 256) {
+    const int lane = c & 63, mt = (c >> 6) & 1, dt = c >> 7;
+    const int ch = 32 * dt + (lane & 31);
+    const float mean = v_mean ? v_mean[ch] : 0.f;
+    const float rc = v_recp[ch];
+    int w[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+      float f[4];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int r = 32 * mt + 8 * g + 4 * (lane >> 5) + q;
+        const float x = F16x<DT>::to_f32(tile[r * PITCH + ch]);
+        f[q] = (tok0 + r < N) ? (x - mean) * rc : 0.f;
+      }
+      int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+      p = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], p, true);
+      w[g] = p;
+    }
+    *reinterpret_cast<v4i*>(ob + (int64_t)c * 16) = v4i{w[0], w[1], w[2], w[3]};
+  }
+}
+
+// where v_fp8_stats leaves recp[b,h,:] inside the partial-sum workspace
+__host__ __device__ inline int64_t v_recp_offset(int64_t bh, int n_chunks, int D) { return bh * n_chunks * 3 * D; }
+
+// per-(batch, head, channel) statistics of V: v_scale = max|v - mean| / 448, v_mean = mean over the
+// N tokens (0 if !smooth), and recp = 448 / max|v - mean| at partial[v_recp_offset(bh, ...) + ch];
+// two launches on `st` (defined in v_fp8.hip)
+int v_fp8_stats(const void* v, int dtype, float* v_scale, float* v_mean, float* partial, int B, int Hkv, int N,
+                int D, int64_t vs_b, int64_t vs_h, int64_t vs_n, int smooth, hipStream_t st);
+
+}  // namespace paro

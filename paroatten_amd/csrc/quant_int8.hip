@@ -5,7 +5,7 @@
 // wave reduction, and the int8 result leaves as 8-byte stores.  Nothing goes through LDS.
 // Arithmetic follows QuantInt8Kernel of the reference (csrc/fused/fused.cu:64-198) in IEEE fp32:
 // this file is compiled without fast-math and with fp contraction off.
-#include "paro_common.hpp"
+#include "paro_device.hpp"
 
 namespace paro {
 
@@ -46,8 +46,7 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(
   // value of element (chunk i, slot j) after mean subtraction / scaling; recomputed in the
   // second pass instead of being kept, so that only the packed input stays in registers
   auto value = [&](int i, int j) -> float {
-    const unsigned w = (unsigned)raw[i][j >> 1];
-    float f = F16x<DT>::to_f32((unsigned short)((j & 1) ? (w >> 16) : (w & 0xffffu)));
+    float f = elem16_to_f32<DT>(raw[i], j);
     if constexpr (MEAN) f -= mv[j];
     if constexpr (SMS) f *= sm_scale;
     return f;
@@ -70,14 +69,13 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(
 #pragma unroll
   for (int i = 0; i < CH; i++) {
     const int tok = g * G + i * ROWS_PER_IT + row0;
-    unsigned w[2] = {0u, 0u};
+    // |value * (127/amax)| <= 127 up to rounding: the reference's clamp to [-128,127] never acts
+    float y[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      float r = rintf(value(i, j) * inv);
-      r = fminf(fmaxf(r, -128.f), 127.f);
-      w[j >> 2] |= ((unsigned)((int)r) & 0xffu) << (8 * (j & 3));
-    }
-    if (tok < N) *reinterpret_cast<v2i*>(ob + (int64_t)tok * os_n) = v2i{(int)w[0], (int)w[1]};
+    for (int j = 0; j < 8; j++) y[j] = value(i, j) * inv;
+    if (tok < N)
+      *reinterpret_cast<v2i*>(ob + (int64_t)tok * os_n) =
+          v2i{(int)pack4_rint_i8(y[0], y[1], y[2], y[3]), (int)pack4_rint_i8(y[4], y[5], y[6], y[7])};
   }
 }
 

@@ -11,36 +11,9 @@
 // (f,h,w) of a head with order p goes to (c[p0]*S[p1] + c[p1])*S[p2] + c[p2].
 // Rotation (diffusers apply_rotary_emb as called at paroattention/cogvideox.py:167-172): fp32
 // products and sum, each rounded (this file is built with fp contraction off).
-#include "paro_common.hpp"
+#include "paro_device.hpp"
 
 namespace paro {
-
-// strides of the (f,h,w) coordinates in the permuted order `order`
-__device__ __forceinline__ void order_strides(int order, int F, int Hh, int W, int& sf, int& sh, int& sw) {
-  switch (order) {
-    default:
-    case 0: sf = Hh * W; sh = W;     sw = 1;      break;  // FHW
-    case 1: sf = W * Hh; sw = Hh;    sh = 1;      break;  // FWH
-    case 2: sh = W * F;  sw = F;     sf = 1;      break;  // HWF
-    case 3: sh = F * W;  sf = W;     sw = 1;      break;  // HFW
-    case 4: sw = Hh * F; sh = F;     sf = 1;      break;  // WHF
-    case 5: sw = F * Hh; sf = Hh;    sh = 1;      break;  // WFH
-  }
-}
-
-template <int DT>
-__device__ __forceinline__ v4i rotate8(const v4i raw, const float* cs, const float* sn) {
-  v4i o;
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    const float x0 = F16x<DT>::to_f32((unsigned short)((unsigned)raw[j] & 0xffffu));
-    const float x1 = F16x<DT>::to_f32((unsigned short)((unsigned)raw[j] >> 16));
-    const float o0 = __fsub_rn(__fmul_rn(x0, cs[2 * j]), __fmul_rn(x1, sn[2 * j]));
-    const float o1 = __fadd_rn(__fmul_rn(x1, cs[2 * j + 1]), __fmul_rn(x0, sn[2 * j + 1]));
-    o[j] = (int)((unsigned)F16x<DT>::from_f32(o0) | ((unsigned)F16x<DT>::from_f32(o1) << 16));
-  }
-  return o;
-}
 
 template <int DT, int D, bool INVERSE>
 __global__ void __launch_bounds__(256) rope_permute_kernel(

@@ -4,17 +4,16 @@
 //
 // Three launches, all HBM-bound and deterministic (no float atomics):
 //   v_stats    : per 256-token chunk, per channel: sum, min, max          (reads V once)
-//   v_finalize : per (b,h,channel): mean = sum/N, scale = max(max-mean, mean-min)/448
-//   v_pack     : per 64-token tile: (v-mean)/scale -> e4m3, fragment order  (reads V once more)
+//   v_finalize : per (b,h,channel): mean = sum/N, amax = max(max-mean, mean-min), scale = amax/448,
+//                recp = 448/amax
+//   v_pack     : per 64-token tile: (v-mean)*recp -> e4m3, fragment order  (reads V once more)
 // max|v-mean| over tokens equals max(max-mean, mean-min) exactly because fp32 subtraction is
 // monotonic, so no second reduction pass is needed.
 // Arithmetic follows MeanScaleKernel of the reference (csrc/fused/fused.cu:316-427) except that the
 // mean divides by the true token count.
-#include "paro_common.hpp"
+#include "paro_device.hpp"
 
 namespace paro {
-
-constexpr int V_CHUNK = 256;  // tokens per stats chunk
 
 template <int DT, int D>
 __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __restrict__ v,
@@ -80,8 +79,7 @@ __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __re
 }
 
 template <int D>
-__global__ void __launch_bounds__(1024) v_finalize_kernel(const float* __restrict__ partial,
-                                                          float* __restrict__ v_scale,
+__global__ void __launch_bounds__(1024) v_finalize_kernel(float* partial, float* __restrict__ v_scale,
                                                           float* __restrict__ v_mean, int N, int n_chunks,
                                                           int smooth) {
   // 1024 / D slices of the chunk range per channel, combined through LDS in a fixed order
@@ -110,14 +108,17 @@ __global__ void __launch_bounds__(1024) v_finalize_kernel(const float* __restric
     const float amax = fmaxf(mx - mean, mean - mn);
     v_scale[bh * D + ch] = amax / 448.0f;
     if (v_mean) v_mean[bh * D + ch] = mean;
+    // every thread of this workgroup has read its partials before the barrier above: the head of the
+    // region is free to carry the reciprocal to the pack kernel
+    partial[v_recp_offset(bh, n_chunks, D) + ch] = amax > 0.f ? 448.0f / amax : 0.f;
   }
 }
 
 template <int DT, int D>
 __global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __restrict__ v,
                                                      uint8_t* __restrict__ v8,
-                                                     const float* __restrict__ v_scale,
-                                                     const float* __restrict__ v_mean, int N, int nb,
+                                                     const float* __restrict__ v_recp,
+                                                     const float* __restrict__ v_mean, int N, int nb, int n_chunks,
                                                      int64_t vs_b, int64_t vs_h, int64_t vs_n) {
   constexpr int LPR = D / 8;
   constexpr int ROWS = 256 / LPR;
@@ -135,44 +136,39 @@ __global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __res
     *reinterpret_cast<v4i*>(&tile[r * PITCH + col]) = raw;
   }
   __syncthreads();
-  uint8_t* ob = v8 + (bh * nb + kb) * (int64_t)(64 * D);
-#pragma unroll
-  for (int c = t; c < 4 * D; c += 256) {  // 16-byte output pieces of this tile
-    const int lane = c & 63, mt = (c >> 6) & 1, dt = c >> 7;
-    const int ch = 32 * dt + (lane & 31);
-    const float mean = v_mean ? v_mean[bh * D + ch] : 0.f;
-    const float sc = v_scale[bh * D + ch];
-    int w[4];
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-      float f[4];
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int r = 32 * mt + 8 * g + 4 * (lane >> 5) + q;
-        const float x = F16x<DT>::to_f32(tile[r * PITCH + ch]);
-        f[q] = (kb * 64 + r < N && sc > 0.f) ? (x - mean) / sc : 0.f;
-      }
-      int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
-      p = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], p, true);
-      w[g] = p;
-    }
-    *reinterpret_cast<v4i*>(ob + (int64_t)c * 16) = v4i{w[0], w[1], w[2], w[3]};
-  }
+  pack_v_tile<DT, D, PITCH>(tile, v8 + (bh * nb + kb) * (int64_t)(64 * D), v_recp + v_recp_offset(bh, n_chunks, D),
+                            v_mean ? v_mean + bh * D : nullptr, kb * 64, N, t);
 }
 
 template <int DT, int D>
-static int run_v_fp8(const void* v, uint8_t* v8, float* v_scale, float* v_mean, float* partial, int B, int Hkv,
-                     int N, int64_t vs_b, int64_t vs_h, int64_t vs_n, int smooth, hipStream_t st) {
-  const int n_chunks = ceil_div(N, V_CHUNK), nb = ceil_div(N, 64);
-  const unsigned short* vp = (const unsigned short*)v;
-  hipLaunchKernelGGL((v_stats_kernel<DT, D>), dim3(n_chunks, Hkv, B), dim3(256), 0, st, vp, partial, N, n_chunks,
-                     vs_b, vs_h, vs_n);
+static int run_v_stats(const void* v, float* v_scale, float* v_mean, float* partial, int B, int Hkv, int N,
+                       int64_t vs_b, int64_t vs_h, int64_t vs_n, int smooth, hipStream_t st) {
+  const int n_chunks = ceil_div(N, V_CHUNK);
+  hipLaunchKernelGGL((v_stats_kernel<DT, D>), dim3(n_chunks, Hkv, B), dim3(256), 0, st, (const unsigned short*)v,
+                     partial, N, n_chunks, vs_b, vs_h, vs_n);
   PARO_HIP(hipGetLastError());
-  hipLaunchKernelGGL((v_finalize_kernel<D>), dim3(B * Hkv), dim3(1024), 0, st, (const float*)partial, v_scale,
-                     v_mean, N, n_chunks, smooth);
+  hipLaunchKernelGGL((v_finalize_kernel<D>), dim3(B * Hkv), dim3(1024), 0, st, partial, v_scale, v_mean, N,
+                     n_chunks, smooth);
   PARO_HIP(hipGetLastError());
-  hipLaunchKernelGGL((v_pack_kernel<DT, D>), dim3(nb, Hkv, B), dim3(256), 0, st, vp, v8,
-                     (const float*)v_scale, (const float*)(smooth ? v_mean : nullptr), N, nb, vs_b, vs_h, vs_n);
+  return PARO_OK;
+}
+
+int v_fp8_stats(const void* v, int dtype, float* v_scale, float* v_mean, float* partial, int B, int Hkv, int N,
+                int D, int64_t vs_b, int64_t vs_h, int64_t vs_n, int smooth, hipStream_t st) {
+  if (dtype == PARO_DTYPE_F16) {
+    if (D == 64) return run_v_stats<PARO_DTYPE_F16, 64>(v, v_scale, v_mean, partial, B, Hkv, N, vs_b, vs_h, vs_n, smooth, st);
+    return run_v_stats<PARO_DTYPE_F16, 128>(v, v_scale, v_mean, partial, B, Hkv, N, vs_b, vs_h, vs_n, smooth, st);
+  }
+  if (D == 64) return run_v_stats<PARO_DTYPE_BF16, 64>(v, v_scale, v_mean, partial, B, Hkv, N, vs_b, vs_h, vs_n, smooth, st);
+  return run_v_stats<PARO_DTYPE_BF16, 128>(v, v_scale, v_mean, partial, B, Hkv, N, vs_b, vs_h, vs_n, smooth, st);
+}
+
+template <int DT, int D>
+static int run_v_pack(const void* v, uint8_t* v8, const float* v_recp, const float* v_mean, int B, int Hkv, int N,
+                      int64_t vs_b, int64_t vs_h, int64_t vs_n, hipStream_t st) {
+  const int nb = ceil_div(N, 64);
+  hipLaunchKernelGGL((v_pack_kernel<DT, D>), dim3(nb, Hkv, B), dim3(256), 0, st, (const unsigned short*)v, v8,
+                     v_recp, v_mean, N, nb, ceil_div(N, V_CHUNK), vs_b, vs_h, vs_n);
   PARO_HIP(hipGetLastError());
   return PARO_OK;
 }
@@ -232,12 +228,16 @@ extern "C" int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_s
              PARO_ERR_RUNTIME, "Tensor value must be 16-byte aligned with strides that are multiples of 8");
   PARO_CHECK(((uintptr_t)v8 % 16) == 0, PARO_ERR_RUNTIME, "paro_v_fp8_pack: v8 must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
+  if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, partial, B, Hkv, N, D, v_stride_b, v_stride_h, v_stride_n,
+                           smooth, st))
+    return rc;
+  const float* mean = smooth ? v_mean : nullptr;
   if (dtype == PARO_DTYPE_F16) {
-    if (D == 64) return run_v_fp8<PARO_DTYPE_F16, 64>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
-    return run_v_fp8<PARO_DTYPE_F16, 128>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
+    if (D == 64) return run_v_pack<PARO_DTYPE_F16, 64>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
+    return run_v_pack<PARO_DTYPE_F16, 128>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
   }
-  if (D == 64) return run_v_fp8<PARO_DTYPE_BF16, 64>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
-  return run_v_fp8<PARO_DTYPE_BF16, 128>(v, v8, v_scale, v_mean, partial, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, smooth, st);
+  if (D == 64) return run_v_pack<PARO_DTYPE_BF16, 64>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
+  return run_v_pack<PARO_DTYPE_BF16, 128>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
 }
 
 extern "C" int paro_sub_mean(const void* v, int dtype, const void* mean, void* out_f16, int B, int H, int N,

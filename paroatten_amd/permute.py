@@ -7,7 +7,7 @@ writes them once, and one launch for the output.  All functions take HND tensors
 """
 from __future__ import annotations
 
-from typing import Optional, Sequence, Tuple
+from typing import NamedTuple, Optional, Sequence, Tuple
 
 import torch
 
@@ -73,6 +73,85 @@ def rope_permute(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Option
         ref.stride(0), ref.stride(1), ref.stride(2), o_ref.stride(0), o_ref.stride(1), o_ref.stride(2),
         stream_of(ref)))
     return tuple(outs)
+
+
+class PreparedOperands(NamedTuple):
+    """What the attention kernel reads: see rope_permute_quant."""
+    q8: torch.Tensor
+    q_scale: torch.Tensor
+    k8: torch.Tensor
+    k_scale: torch.Tensor
+    v8: torch.Tensor
+    v_scale: torch.Tensor
+    v_mean: Optional[torch.Tensor]
+
+
+def _tables_ok(cos, sin, n_img, D):
+    if cos is None:
+        return
+    for t, n in ((cos, "cos"), (sin, "sin")):
+        _lib.require_gpu(t, n)
+        if t.dtype != torch.float32 or tuple(t.shape) != (n_img, D) or not t.is_contiguous():
+            raise RuntimeError(f"Tensor {n} must be contiguous float32 of shape ({n_img}, {D})")
+
+
+def rope_k_mean(k: torch.Tensor, grid: Sequence[int], n_text: int, cos: Optional[torch.Tensor] = None,
+                sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[B,H,1,D] in k's dtype: the token mean of K after the rotation, i.e. the `km` the reference's
+    quantiser expects (paroattention/quant.py:105-180) when it runs behind the processor's RoPE."""
+    _check_hnd(k, "key")
+    B, H, N, D = k.shape
+    F, Hh, W = (int(x) for x in grid)
+    _tables_ok(cos, sin, F * Hh * W, D)
+    lib = load()
+    km = torch.empty((B, H, 1, D), dtype=k.dtype, device=k.device)
+    ws = torch.empty(int(lib.paro_prep_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=k.device)
+    check(lib.paro_rope_k_mean(ptr(k), _lib.DTYPE_CODE[k.dtype], ptr(cos), ptr(sin), ptr(km), ptr(ws), ws.numel(),
+                               B, H, N, D, int(n_text), F, Hh, W, k.stride(0), k.stride(1), k.stride(2),
+                               km.stride(0), km.stride(1), stream_of(k)))
+    return km
+
+
+def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders: torch.Tensor,
+                       grid: Sequence[int], n_text: int, cos: Optional[torch.Tensor] = None,
+                       sin: Optional[torch.Tensor] = None, km: Optional[torch.Tensor] = None,
+                       smooth_v: bool = True) -> PreparedOperands:
+    """rope_permute + per_warp_int8(BLKQ=64, WARPQ=32, BLKK=64, km) + per_channel_fp8 in one pass, with
+    bit-identical INT8 results and without the permuted 16-bit tensors ever being written.  q, k, v:
+    [B,H,N,D] views with equal strides (e.g. the transposed token-major projections); km: None or
+    [B,H,1,D] in the input dtype (see rope_k_mean)."""
+    _check_hnd(q, "query")
+    B, H, N, D = q.shape
+    for t, n in ((k, "key"), (v, "value")):
+        _check_hnd(t, n)
+        if t.shape != q.shape or t.stride() != q.stride() or t.dtype != q.dtype:
+            raise RuntimeError("q, k, v must share shape, strides and dtype")
+    _check_orders(orders, H)
+    F, Hh, W = (int(x) for x in grid)
+    _tables_ok(cos, sin, F * Hh * W, D)
+    ms_b = ms_h = 0
+    if km is not None:
+        _lib.require_gpu(km, "km")
+        if km.dtype != q.dtype or tuple(km.shape) != (B, H, 1, D) or km.stride(-1) != 1:
+            raise RuntimeError(f"Tensor km must have shape ({B}, {H}, 1, {D}) and the dtype of key")
+        ms_b, ms_h = km.stride(0), km.stride(1)
+    lib = load()
+    dev = q.device
+    nb = (N + 63) // 64
+    q8 = torch.empty((B, H, N, D), dtype=torch.int8, device=dev)
+    k8 = torch.empty((B, H, N, D), dtype=torch.int8, device=dev)
+    q_scale = torch.empty((B, H, nb * 2), dtype=torch.float32, device=dev)
+    k_scale = torch.empty((B, H, nb), dtype=torch.float32, device=dev)
+    v8 = torch.empty(int(lib.paro_v_fp8_bytes(B, H, N, D)), dtype=torch.uint8, device=dev)
+    v_scale = torch.empty((B, H, D), dtype=torch.float32, device=dev)
+    v_mean = torch.empty((B, H, D), dtype=torch.float32, device=dev)
+    ws = torch.empty(int(lib.paro_prep_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=dev)
+    check(lib.paro_rope_permute_quant_fwd(
+        ptr(q), ptr(k), ptr(v), _lib.DTYPE_CODE[q.dtype], ptr(cos), ptr(sin), ptr(orders), ptr(km),
+        ptr(q8), ptr(q_scale), ptr(k8), ptr(k_scale), ptr(v8), ptr(v_scale), ptr(v_mean), ptr(ws), ws.numel(),
+        B, H, N, D, int(n_text), F, Hh, W, q.stride(0), q.stride(1), q.stride(2), ms_b, ms_h,
+        1 if smooth_v else 0, stream_of(q)))
+    return PreparedOperands(q8, q_scale, k8, k_scale, v8, v_scale, v_mean if smooth_v else None)
 
 
 def permute_inverse(o: torch.Tensor, orders: torch.Tensor, grid: Sequence[int], n_text: int,
