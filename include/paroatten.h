@@ -175,7 +175,7 @@ int paro_permute_index_map(int32_t* idx, const int32_t* orders, int H, int F, in
  * order, so it may differ in the last fp32 bit), i.e. as what the processors do between the projections and the
  * attention call (paroattention/cogvideox.py:167-186 with quant.py:105-180 and, for V,
  * quant.py:224-293), without writing the permuted 16-bit tensors.
- * q, k, v: [B,H,N,D] through the three input strides (shared by the three tensors).  k_mean: NULL
+ * q, k, v: [B,H,N,D], each through its own three strides.  k_mean: NULL
  * or [B,H,D] in the input dtype through mean strides (subtracted from the rotated K before
  * quantisation).  Outputs, all contiguous: q8, k8 int8 [B,H,N,D]; q_scale f32 [B,H,2*ceil(N/64)];
  * k_scale f32 [B,H,ceil(N/64)]; v8 paro_v_fp8_bytes(); v_scale, v_mean f32 [B,H,D].
@@ -191,7 +191,9 @@ int paro_rope_permute_quant_fwd(const void* q, const void* k, const void* v, int
                                 uint8_t* v8, float* v_scale, float* v_mean,
                                 void* workspace, int64_t workspace_bytes,
                                 int B, int H, int N, int D, int n_text, int F, int Hh, int W,
-                                int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_n,
+                                int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                                int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
                                 int64_t mean_stride_b, int64_t mean_stride_h,
                                 int smooth_v, void* stream);
 int paro_rope_k_mean(const void* k, int dtype, const float* cos, const float* sin, void* k_mean,

@@ -51,7 +51,8 @@ SIGNATURES = {
     "paro_permute_index_map": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
     "paro_prep_workspace_bytes": (c_int64, [_I, _I, _I, _I]),
     "paro_rope_permute_quant_fwd": (c_int, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L,
-                                            _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _I, _P]),
+                                            _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _L,
+                                            _L, _L, _I, _P]),
     "paro_rope_k_mean": (c_int, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _I,
                                  _L, _L, _L, _L, _L, _P]),
     "paro_mask_bits_bytes": (c_int64, [_L]),

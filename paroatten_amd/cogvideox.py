@@ -4,10 +4,10 @@
 `PARO_CogVideoXAttnProcessor2_0` keeps the reference's constructor, injected attributes
 (`permute_plan`, `i_block`, `i_timestep`, and `sparse_mask` or `prefetch_stream`), call signature,
 return value and `get_time_stats()`.  What changes underneath:
-  * RoPE and the per-head permutation of Q, K, V are one launch that reads the projections in
-    their native token-major memory ([B,N,H*D] viewed as [B,H,N,D] through strides): no
-    transpose copy, no in-place rotate pass, no Python loop over heads, no host sync;
-  * V stays bf16/fp16 (the FP8 conversion is inside the attention entry point);
+  * RoPE, the per-head permutation of Q, K, V, the INT8 quantisation of Q/K and the FP8 packing of V
+    are one pass that reads the projections in their native token-major memory ([B,N,H*D] viewed as
+    [B,H,N,D] through strides) and writes only what the attention kernel reads: no transpose copy,
+    no in-place rotate pass, no Python loop over heads, no host sync, no `.to(float16)` of V;
   * the inverse permutation writes token-major memory directly, so the reshape for the output
     projection is a view;
   * (F,H,W), literals in the reference (cogvideox.py:31-33), are the `grid` argument/attribute;
@@ -23,7 +23,7 @@ import torch.nn.functional as F
 from . import _qattn_sm80 as qattn
 from . import permute as PM
 from .permute import permute_attn_out, permute_qk  # noqa: F401  (same module-level names as the reference)
-from .quant import per_warp_int8 as per_warp_int8_cuda
+from .quant import per_warp_int8 as per_warp_int8_cuda  # noqa: F401  (the reference's module-level name)
 
 COG_GRID = (13, 30, 45)   # frames x height x width of CogVideoX-5b latents after patching (cogvideox.py:31-33)
 
@@ -115,12 +115,20 @@ class _ParoProcessorBase:
         _, _, vp = PM.rope_permute(None, None, value, orders, grid, n_text)
         return qp, kp, vp
 
-    def _sparse_attention(self, qp, kp, vp, sm_scale):
-        km = kp.mean(dim=2, keepdim=True) if self.smooth_k else None
-        q8, qs, k8, ks = per_warp_int8_cuda(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64, tensor_layout="HND")
-        out = torch.empty_like(qp)
-        qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, vp, out, qs, ks, 1, 0, 2, sm_scale, 0, self._mask(),
-                                            exact_exp=self.exact_exp)
+    def _prepare(self, query, key, value, orders, grid, n_text, cos, sin, rotate_key=True):
+        """RoPE + permutation + INT8 Q/K + FP8 V in one pass, straight from the projections."""
+        if not rotate_key and cos is not None:
+            # keys that must not be rotated: rotate the queries separately, then prepare without tables
+            query, _, _ = PM.rope_permute(query, None, None, torch.zeros_like(orders), grid, n_text, cos, sin)
+            cos = sin = None
+        km = PM.rope_k_mean(key, grid, n_text, cos, sin) if self.smooth_k else None
+        return PM.rope_permute_quant(query, key, value, orders, grid, n_text, cos, sin, km=km)
+
+    def _sparse_attention(self, ops, dtype, sm_scale):
+        B, H, N, D = ops.q8.shape
+        out = torch.empty((B, H, N, D), dtype=dtype, device=ops.q8.device)
+        qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, out, ops.q_scale, ops.k_scale,
+                                    sm_scale, self._mask(), exact_exp=self.exact_exp)
         return out
 
     def get_time_stats(self):
@@ -170,14 +178,12 @@ class PARO_CogVideoXAttnProcessor2_0(_ParoProcessorBase):
             orders = torch.zeros(attn.heads, dtype=torch.int32, device=query.device)   # order 0 = identity
         else:
             orders = self._orders(query.device)
-        # keys of a cross-attention layer are not rotated (cogvideox.py:170-172)
-        qp, kp, vp = self._rope_permute(query, key, value, orders, grid, text_seq_length, cos, sin,
-                                        rotate_key=not getattr(attn, "is_cross_attention", False))
-
+        rotate_key = not getattr(attn, "is_cross_attention", False)   # cogvideox.py:170-172
         done = self._timer.start()
         token_major = torch.empty((batch_size, sequence_length, attn.heads, head_dim), dtype=query.dtype,
                                   device=query.device)
         if dense:
+            qp, kp, vp = self._rope_permute(query, key, value, orders, grid, text_seq_length, cos, sin, rotate_key)
             if attention_mask is not None:
                 attention_mask = attn.prepare_attention_mask(attention_mask, sequence_length, batch_size)
                 attention_mask = attention_mask.view(batch_size, attn.heads, -1, attention_mask.shape[-1])
@@ -185,7 +191,8 @@ class PARO_CogVideoXAttnProcessor2_0(_ParoProcessorBase):
             token_major.copy_(out.transpose(1, 2))
             done.record()
         else:
-            out = self._sparse_attention(qp, kp, vp, 1.0 / (head_dim ** 0.5))
+            ops = self._prepare(query, key, value, orders, grid, text_seq_length, cos, sin, rotate_key)
+            out = self._sparse_attention(ops, query.dtype, 1.0 / (head_dim ** 0.5))
             done.record()
             PM.permute_inverse(out, orders, grid, text_seq_length, out=token_major.transpose(1, 2))
         self.call_count += 1

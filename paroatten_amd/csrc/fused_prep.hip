@@ -53,7 +53,8 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
     const int* __restrict__ orders, const unsigned short* __restrict__ k_mean, int8_t* __restrict__ q8,
     float* __restrict__ q_scale, int8_t* __restrict__ k8, float* __restrict__ k_scale, uint8_t* __restrict__ v8,
     const float* __restrict__ v_recp, const float* __restrict__ v_mean, int BH, int H, int N, int nb, int n_text,
-    int F, int Hh, int W, int head_split, int64_t is_b, int64_t is_h, int64_t is_n, int64_t ms_b, int64_t ms_h) {
+    int F, int Hh, int W, int head_split, int64_t qs_b, int64_t qs_h, int64_t qs_n, int64_t ks_b, int64_t ks_h,
+    int64_t ks_n, int64_t vs_b, int64_t vs_h, int64_t vs_n, int64_t ms_b, int64_t ms_h) {
   constexpr int LPR = D / 8;            // lanes per token row (16-byte pieces)
   constexpr int RPI = 64 / LPR;         // rows one wave covers per load instruction
   constexpr int PC = 16 / RPI;          // pieces per lane: a wave owns 16 rows of the block
@@ -102,8 +103,6 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
     const int b = bh / H, head = bh - b * H;
     if (orders[head] != order) continue;                  // uniform over the workgroup
     if ((n_match++ % head_split) != split) continue;
-    const int64_t in_base = b * is_b + head * is_h;
-
     float mv[8];
     if (k_mean) {
       const v4i m = *reinterpret_cast<const v4i*>(k_mean + b * ms_b + head * ms_h + col);
@@ -122,10 +121,9 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
       rq[i] = rv;
       rk[i] = rv;
       if (src[i] >= 0) {
-        const int64_t o = in_base + (int64_t)src[i] * is_n + col;
-        rq[i] = *reinterpret_cast<const v4i*>(q_in + o);
-        rk[i] = *reinterpret_cast<const v4i*>(k_in + o);
-        rv = *reinterpret_cast<const v4i*>(v_in + o);
+        rq[i] = *reinterpret_cast<const v4i*>(q_in + b * qs_b + head * qs_h + (int64_t)src[i] * qs_n + col);
+        rk[i] = *reinterpret_cast<const v4i*>(k_in + b * ks_b + head * ks_h + (int64_t)src[i] * ks_n + col);
+        rv = *reinterpret_cast<const v4i*>(v_in + b * vs_b + head * vs_h + (int64_t)src[i] * vs_n + col);
       }
       *reinterpret_cast<v4i*>(&s_tile[(row0 + i * RPI) * PITCH + col]) = rv;
     }
@@ -335,13 +333,18 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
                                            int8_t* q8, float* q_scale, int8_t* k8, float* k_scale, uint8_t* v8,
                                            float* v_scale, float* v_mean, void* workspace, int64_t workspace_bytes,
                                            int B, int H, int N, int D, int n_text, int F, int Hh, int W,
-                                           int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_n,
+                                           int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                                           int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                           int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
                                            int64_t mean_stride_b, int64_t mean_stride_h, int smooth_v,
                                            void* stream) {
   using namespace paro;
-  if (int rc = check_prep("paro_rope_permute_quant_fwd", dtype, B, H, N, D, n_text, F, Hh, W, in_stride_b,
-                          in_stride_h, in_stride_n))
+  if (int rc = check_prep("paro_rope_permute_quant_fwd", dtype, B, H, N, D, n_text, F, Hh, W, q_stride_b,
+                          q_stride_h, q_stride_n))
     return rc;
+  PARO_CHECK(k_stride_b % 8 == 0 && k_stride_h % 8 == 0 && k_stride_n % 8 == 0 && v_stride_b % 8 == 0 &&
+                 v_stride_h % 8 == 0 && v_stride_n % 8 == 0,
+             PARO_ERR_RUNTIME, "paro_rope_permute_quant_fwd: strides must be multiples of 8 elements");
   PARO_CHECK(q && k && v && orders && q8 && q_scale && k8 && k_scale && v8 && v_scale && workspace, PARO_ERR_RUNTIME,
              "paro_rope_permute_quant_fwd: null pointer");
   PARO_CHECK(!smooth_v || v_mean, PARO_ERR_RUNTIME, "paro_rope_permute_quant_fwd: smoothing needs a v_mean buffer");
@@ -358,8 +361,8 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
              (long long)workspace_bytes);
   hipStream_t st = (hipStream_t)stream;
   // V statistics do not depend on the token order: taken on the unpermuted tensor
-  if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, (float*)workspace, B, H, N, D, in_stride_b, in_stride_h,
-                           in_stride_n, smooth_v, st))
+  if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, (float*)workspace, B, H, N, D, v_stride_b, v_stride_h,
+                           v_stride_n, smooth_v, st))
     return rc;
   const int nb = ceil_div(N, 64);
   // every order gets `head_split` workgroups per block, each walking over its share of the (batch,
@@ -373,7 +376,8 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
                      (const unsigned short*)k, (const unsigned short*)v, cos, sin, (const int*)orders,          \
                      (const unsigned short*)k_mean, q8, q_scale, k8, k_scale, v8, (const float*)workspace,      \
                      (const float*)(smooth_v ? v_mean : nullptr), B * H, H, N, nb, n_text, F, Hh, W, head_split, \
-                     in_stride_b, in_stride_h, in_stride_n, mean_stride_b, mean_stride_h)
+                     q_stride_b, q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n, v_stride_b,        \
+                     v_stride_h, v_stride_n, mean_stride_b, mean_stride_h)
   if (dtype == PARO_DTYPE_F16) {
     if (D == 64) PARO_PREP(PARO_DTYPE_F16, 64); else PARO_PREP(PARO_DTYPE_F16, 128);
   } else {

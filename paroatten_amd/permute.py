@@ -118,14 +118,14 @@ def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders
                        smooth_v: bool = True) -> PreparedOperands:
     """rope_permute + per_warp_int8(BLKQ=64, WARPQ=32, BLKK=64, km) + per_channel_fp8 in one pass, with
     bit-identical INT8 results and without the permuted 16-bit tensors ever being written.  q, k, v:
-    [B,H,N,D] views with equal strides (e.g. the transposed token-major projections); km: None or
+    [B,H,N,D] views, each with its own strides (e.g. the transposed token-major projections); km: None or
     [B,H,1,D] in the input dtype (see rope_k_mean)."""
     _check_hnd(q, "query")
     B, H, N, D = q.shape
     for t, n in ((k, "key"), (v, "value")):
         _check_hnd(t, n)
-        if t.shape != q.shape or t.stride() != q.stride() or t.dtype != q.dtype:
-            raise RuntimeError("q, k, v must share shape, strides and dtype")
+        if t.shape != q.shape or t.dtype != q.dtype:
+            raise RuntimeError("q, k, v must share shape and dtype")
     _check_orders(orders, H)
     F, Hh, W = (int(x) for x in grid)
     _tables_ok(cos, sin, F * Hh * W, D)
@@ -149,8 +149,8 @@ def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders
     check(lib.paro_rope_permute_quant_fwd(
         ptr(q), ptr(k), ptr(v), _lib.DTYPE_CODE[q.dtype], ptr(cos), ptr(sin), ptr(orders), ptr(km),
         ptr(q8), ptr(q_scale), ptr(k8), ptr(k_scale), ptr(v8), ptr(v_scale), ptr(v_mean), ptr(ws), ws.numel(),
-        B, H, N, D, int(n_text), F, Hh, W, q.stride(0), q.stride(1), q.stride(2), ms_b, ms_h,
-        1 if smooth_v else 0, stream_of(q)))
+        B, H, N, D, int(n_text), F, Hh, W, q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1),
+        k.stride(2), v.stride(0), v.stride(1), v.stride(2), ms_b, ms_h, 1 if smooth_v else 0, stream_of(q)))
     return PreparedOperands(q8, q_scale, k8, k_scale, v8, v_scale, v_mean if smooth_v else None)
 
 

@@ -95,16 +95,16 @@ class PARO_WanAttnProcessor2_0(_ParoProcessorBase):
             orders = self._orders(query.device)
         else:
             orders = torch.zeros(attn.heads, dtype=torch.int32, device=query.device)   # order 0 = identity
-        qp, kp, vp = self._rope_permute(query, key, value, orders, grid, 0, cos, sin)
-
         done = self._timer.start()
         token_major = torch.empty((batch_size, sequence_length, attn.heads, head_dim), dtype=query.dtype,
                                   device=query.device)
         if sparse:
-            out = self._sparse_attention(qp, kp, vp, 1.0 / (head_dim ** 0.5))
+            ops = self._prepare(query, key, value, orders, grid, 0, cos, sin)
+            out = self._sparse_attention(ops, query.dtype, 1.0 / (head_dim ** 0.5))
             done.record()
             PM.permute_inverse(out, orders, grid, 0, out=token_major.transpose(1, 2))
         else:
+            qp, kp, vp = self._rope_permute(query, key, value, orders, grid, 0, cos, sin)
             out = F.scaled_dot_product_attention(qp, kp, vp, attn_mask=attention_mask, dropout_p=0.0, is_causal=False)
             token_major.copy_(out.transpose(1, 2))
             done.record()

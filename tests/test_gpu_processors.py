@@ -97,7 +97,7 @@ def _cog_case(dev, dtype=torch.bfloat16, seed=0):
     return attn, hidden, text, (cos, sin), masks, plan, grid, n_text
 
 
-def _cog_expected(attn, hidden, text, rotary, mask, plan, i_block, grid, n_text):
+def _cog_expected(attn, hidden, text, rotary, mask, plan, i_block, grid, n_text, smooth_k=False):
     """The reference's sequence (cogvideox.py:139-235) with the oracle in place of the kernels."""
     hs = torch.cat([text, hidden], dim=1)
     B, N, _ = hs.shape
@@ -106,21 +106,22 @@ def _cog_expected(attn, hidden, text, rotary, mask, plan, i_block, grid, n_text)
     k = attn.norm_k(attn.to_k(hs).view(B, N, H, -1).transpose(1, 2))
     v = attn.to_v(hs).view(B, N, H, -1).transpose(1, 2)
     o = O.paro_path(q.cpu().contiguous(), k.cpu().contiguous(), v.cpu().contiguous(), mask[None].expand(B, -1, -1, -1), plan, i_block,
-                    grid, n_text, rotary[0], rotary[1], smooth_k=False)
+                    grid, n_text, rotary[0], rotary[1], smooth_k=smooth_k)
     o = o.to(hs.device).transpose(1, 2).reshape(B, N, -1).to(hs.dtype)
     o = attn.to_out[1](attn.to_out[0](o))
     return o[:, n_text:], o[:, :n_text], q, k, v
 
 
 @torch.no_grad()
-def test_cogvideox_processor_against_oracle(dev):
+@pytest.mark.parametrize("smooth_k", [False, True])
+def test_cogvideox_processor_against_oracle(dev, smooth_k):
     from paroatten_amd import PARO_CogVideoXAttnProcessor2_0
     attn, hidden, text, rotary, masks, plan, grid, n_text = _cog_case(dev)
-    proc = PARO_CogVideoXAttnProcessor2_0(grid=grid)
+    proc = PARO_CogVideoXAttnProcessor2_0(grid=grid, smooth_k=smooth_k)
     proc.permute_plan, proc.i_block, proc.i_timestep = plan, 1, 1
     proc.sparse_mask = masks.to(dev)
     out_h, out_t = proc(attn, hidden, text, image_rotary_emb=(rotary[0].to(dev), rotary[1].to(dev)))
-    ref_h, ref_t, *_ = _cog_expected(attn, hidden, text, rotary, masks[1, 1], plan, 1, grid, n_text)
+    ref_h, ref_t, *_ = _cog_expected(attn, hidden, text, rotary, masks[1, 1], plan, 1, grid, n_text, smooth_k)
     assert out_h.shape == hidden.shape and out_t.shape == text.shape and out_h.dtype == hidden.dtype
     for got, ref in ((out_h, ref_h), (out_t, ref_t)):
         assert cosine(got.cpu(), ref.cpu()) >= 0.999
