@@ -10,7 +10,8 @@ banded-plus-random 64x64 block masks.  One step = one call of the reference's ex
 V -> FP8 tile packing followed by the block-sparse INT8-QK / FP8-PV attention kernel, inputs already
 resident in HBM.  `value` is the reference's "effective" figure 4*B*H*D*N^2 / t (dense-equivalent,
 not scaled by density); `densities` repeats the measurement at 0.5 / 0.3 / 0.2 and `path` times the
-other kernels of the path (fused RoPE+permutation, INT8 quantisation, inverse permutation).
+other kernels of the path (the one-pass preparation RoPE + permutation + INT8 + FP8, the separate
+kernels it replaces, the inverse permutation) and the processors' whole per-layer sequence.
 
 `roofline` is for the attention kernel alone: executed MFMA work 4*64*64*D per kept block, divided
 by the kernel's mean duration between HIP events recorded on the launch stream, against the 5.0
@@ -122,7 +123,7 @@ def main():
     else:
         cos, sin = rope_table_wan_real(D, wl.grid, device=dev)
     qp, kp, vp = PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin)
-    km = kp.mean(dim=2, keepdim=True)
+    km = PM.rope_k_mean(k, wl.grid, wl.n_text, cos, sin)
     q8, qs, k8, ks = Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64)
     out = torch.empty_like(q)
     ws = torch.empty(qattn.workspace_bytes(B, H, N, D), dtype=torch.uint8, device=dev)
@@ -192,13 +193,30 @@ def main():
             path[name] = {"ms": round(t, 4), "GBps": round(nbytes / t / 1e6, 1)}
             path[name]["frac_hbm_peak"] = round(path[name]["GBps"] / PEAK_HBM_GBS, 3)
 
-        timed("rope_permute_qkv", lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), 3 * 2 * el * 2)
-        timed("rope_permute_qk", lambda: PM.rope_permute(q, k, None, orders, wl.grid, wl.n_text, cos, sin), 2 * 2 * el * 2)
+        # one pass from the projections to the attention operands: reads Q, K once and V twice (statistics,
+        # then packing), writes q8, k8, v8
+        timed("prepare_fused_rope_permute_quant_fp8",
+              lambda: PM.rope_permute_quant(q, k, v, orders, wl.grid, wl.n_text, cos, sin, km=km), el * (2 + 2 + 4) + el * 3)
+        timed("rope_k_mean", lambda: PM.rope_k_mean(k, wl.grid, wl.n_text, cos, sin), el * 2)
         timed("permute_inverse_o", lambda: PM.permute_inverse(out, orders, wl.grid, wl.n_text), 2 * el * 2)
+        # the same work as separate kernels (what the fused pass replaces)
+        timed("rope_permute_qkv", lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), 3 * 2 * el * 2)
         timed("quant_int8_qk", lambda: Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64), 2 * el * 3)
         timed("v_fp8_pack", lambda: Q.per_channel_fp8(vp), el * 5)
         # plain device copy of one tensor: what this box sustains for the simplest read+write
         timed("hbm_copy_reference", lambda: out.copy_(q), 2 * el * 2)
+
+        # the processors' whole sequence per layer at the headline density
+        def whole_path():
+            kmean = PM.rope_k_mean(k, wl.grid, wl.n_text, cos, sin)
+            ops = PM.rope_permute_quant(q, k, v, orders, wl.grid, wl.n_text, cos, sin, km=kmean)
+            qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, out, ops.q_scale,
+                                        ops.k_scale, sm_scale, head_mask)
+            PM.permute_inverse(out, orders, wl.grid, wl.n_text)
+
+        t_path = event_time_ms(whole_path, reps, 2)
+        path["whole_path_k_mean_prepare_attention_inverse"] = {
+            "ms": round(t_path, 4), "effective_tops": round(dense_ops / (t_path * 1e-3) / 1e12, 1)}
 
     result = {
         "metric": "effective attn TOPS & %MFMA peak @CogVideoX-5b shape, density 0.2/0.3/0.5",

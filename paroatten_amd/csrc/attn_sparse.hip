@@ -60,7 +60,6 @@ constexpr float P_HEADROOM = 3.75f;
 constexpr int S_MAGIC_BITS = 0x4B400000;  // float 1.5 * 2^23
 constexpr float S_MAGIC_F = 12582912.0f;
 constexpr int FP8_ONES = 0x38383838;  // four e4m3 1.0
-constexpr int NST = 3;                // LDS ring stages
 constexpr float FAST_EXP_SHIFT = -0.35f;  // centres the linear-mantissa error of the fast exponential
 
 __device__ __forceinline__ float max3(float a, float b, float c) {
@@ -111,6 +110,10 @@ __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, int vo
 }
 
 template <int D> struct AttnLds {
+  // LDS ring stages per operand.  D = 64: three, tiles are requested two iterations ahead.  D = 128:
+  // two, requested one iteration ahead (an iteration is twice as long there), which keeps a workgroup
+  // at 32 KB + lists so that four of them, the register-limited number, fit a CU's 160 KB.
+  static constexpr int NST = D == 128 ? 2 : 3;
   static constexpr int KTILE = 64 * D;   // bytes of one K8 tile: 64 rows of D bytes, 16-byte chunks XOR-swizzled
   static constexpr int VTILE = 64 * D;   // bytes of one V8 tile (fragment order, as in HBM)
   static constexpr int V_OFF = NST * KTILE;
@@ -332,17 +335,27 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
   int kb_1 = __builtin_amdgcn_readfirstlane((int)klist[1]);
   int kb_2 = __builtin_amdgcn_readfirstlane((int)klist[2]);
   int kb_3 = __builtin_amdgcn_readfirstlane((int)klist[3]);
+  constexpr bool RING2 = Lds::NST == 2;
   load_k(kb_c, 0);
-  load_v(kb_c, 0);
-  load_v(kb_c, 2);  // the first iteration multiplies this stage by an all-zero P: it must hold finite values
   load_k(kb_1, 1);
-  load_k(kb_2, 2);
+  if constexpr (RING2) {
+    // stage of block j: j % 2.  Iteration i: DMA K(i+2) and V(i) | reads K(i+1), V(i-1); everything an
+    // iteration requests has landed by the barrier at its end
+    load_v(kb_c, 1);  // the first iteration multiplies this stage by an all-zero P: it must hold finite values
+  } else {
+    load_v(kb_c, 0);
+    load_v(kb_c, 2);  // as above
+    load_k(kb_2, 2);
+  }
   float c_cur = qsc * clist[0];
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   read_k_frags(0);
   qk_mfma();
   dump_s(kb_c);
+  // stage 0 is the first one the loop refills: both waves must hold their K(0) fragments by then
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
   v8i pf_a = {0, 0, 0, 0, 0, 0, 0, 0}, pf_b = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // the pending product O^T += V8^T(prev) . P~^T(prev), plus the row sums of the ROUNDED P~ from one
@@ -373,8 +386,13 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
   // left (sk0).
   auto step = [&](int it, int sk0, int sk1, int svp, int sv1, v8i& pf, v8i& pf_p) {
     // -- memory traffic of this iteration, issued up front
-    load_k(kb_3, sk0);
-    load_v(kb_1, sv1);
+    if constexpr (RING2) {
+      load_k(kb_2, sk0);   // K(it+2) into the stage K(it) has left
+      load_v(kb_c, sk0);   // V(it) into the stage V(it-2) has left
+    } else {
+      load_k(kb_3, sk0);
+      load_v(kb_1, sv1);
+    }
     const int kidx_v = (int)klist[it + 4];
     read_v_frags(svp);
     const float c_next = qsc * clist[it + 1];
@@ -521,25 +539,38 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     //    publishes it; this iteration's own DMA may stay in flight
     const int kb_4 = __builtin_amdgcn_readfirstlane(kidx_v);
     // (a bare s_barrier: __syncthreads() would add a fence that waits for ALL outstanding loads)
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS_PER_IT) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(RING2 ? 0 : LOADS_PER_IT) : "memory");
     __builtin_amdgcn_s_barrier();
     kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3; kb_3 = kb_4;
     c_cur = c_next;
   };
 
-  // stage of block j is j % 3: with i = it % 3 the step writes K stage i, reads K stage i+1, reads V
-  // stage i-1 and writes V stage i+1
-  int i3 = 0;  // it % 3
-  for (int it = 0; it < cnt; it += 2) {
-    const int s1 = i3 == 2 ? 0 : i3 + 1, s2 = i3 == 0 ? 2 : i3 - 1;  // (i3+1)%3, (i3+2)%3 == (i3-1)%3
-    step(it, i3, s1, s2, s1, pf_a, pf_b);
-    if (it + 1 >= cnt) { i3 = s1; break; }
-    step(it + 1, s1, s2, i3, s2, pf_b, pf_a);
-    i3 = s2;
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // DMA of the padded tail blocks: nobody reads it
-  // the last block's P.V is still pending: i3 is now cnt % 3, its V tile sits in stage (cnt-1) % 3
-  {
+  if constexpr (RING2) {
+    // stage of block j is j % 2: the step refills stage it % 2 and reads K(it+1), V(it-1) from the other
+    for (int it = 0; it < cnt; it += 2) {
+      step(it, 0, 1, 1, 0, pf_a, pf_b);
+      if (it + 1 >= cnt) break;
+      step(it + 1, 1, 0, 0, 1, pf_b, pf_a);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the last block's P.V is still pending; its V tile sits in stage (cnt-1) % 2
+    read_v_frags((cnt - 1) & 1);
+    const v8i& pf_last = (cnt & 1) ? pf_a : pf_b;
+#pragma unroll
+    for (int i = 0; i < N_PV; i++) pv_one(pf_last, i);
+  } else {
+    // stage of block j is j % 3: with i = it % 3 the step writes K stage i, reads K stage i+1, reads V
+    // stage i-1 and writes V stage i+1
+    int i3 = 0;  // it % 3
+    for (int it = 0; it < cnt; it += 2) {
+      const int s1 = i3 == 2 ? 0 : i3 + 1, s2 = i3 == 0 ? 2 : i3 - 1;  // (i3+1)%3, (i3+2)%3 == (i3-1)%3
+      step(it, i3, s1, s2, s1, pf_a, pf_b);
+      if (it + 1 >= cnt) { i3 = s1; break; }
+      step(it + 1, s1, s2, i3, s2, pf_b, pf_a);
+      i3 = s2;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // DMA of the padded tail blocks: nobody reads it
+    // the last block's P.V is still pending: i3 is now cnt % 3, its V tile sits in stage (cnt-1) % 3
     read_v_frags(i3 == 0 ? 2 : i3 - 1);
     const v8i& pf_last = (cnt & 1) ? pf_a : pf_b;
 #pragma unroll
