@@ -34,10 +34,10 @@ PEAK_MFMA_TOPS = 5000.0  # dense INT8 / FP8 MFMA peak of MI355X, TOP/s
 PEAK_HBM_GBS = 8000.0
 HEADLINE_DENSITY = 0.3
 DENSITIES = (0.5, 0.3, 0.2)
-# HBM bytes per attention-kernel launch at density 0.3 from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/attn_sparse_cogvideox5b_pmc.txt): FETCH_SIZE 164683 x 2.0 KiB + WRITE_SIZE 213341 x 1.0 KiB,
-# the factors being what the same counters read for a plain copy of known size
-ATTN_TRAFFIC_BYTES = int((164683 * 2.0 + 213341 * 1.0) * 1024)
+# HBM bytes per attention-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/path_kernels_cogvideox5b_hbm_traffic.txt): FETCH_SIZE 165562 x 2.0 KiB + WRITE_SIZE 213668 x 1.0 KiB,
+# the factors being what the same counters read for a plain copy of known size; the same at every density
+ATTN_TRAFFIC_BYTES = int((165562 * 2.0 + 213668 * 1.0) * 1024)
 
 
 def event_time_ms(fn, reps, warmup):
@@ -173,13 +173,13 @@ def main():
     hk = dens[str(HEADLINE_DENSITY)]
     achieved = hk["executed_tops_kernel"]
     roofline = {
-        "kernel": "attn_sparse_kernel<64>",
+        "kernel": f"attn_sparse_kernel<{D}>",
         "bound": "mfma",
         "achieved": achieved,
         "peak": PEAK_MFMA_TOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_MFMA_TOPS, 4),
-        "traffic": ATTN_TRAFFIC_BYTES,
+        "traffic": ATTN_TRAFFIC_BYTES if args.workload == "cogvideox5b" else None,
         "ops_per_launch": hk["kept_blocks"] * 4.0 * 64 * 64 * D,
         "avg_launch_ms": hk["attn_kernel_ms"],
     }
