@@ -114,6 +114,25 @@ int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
                          int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
                          float sm_scale, int is_causal, int flags, void* stream);
 
+/* (2b') The same kernel with the inverse token permutation folded into its stores: q-row r of head
+ * `head` is written at token n_text + old(r - n_text), old() = the inverse of the index law of (3)
+ * below for order orders[head] (rows below n_text stay in place).  Stands in for the attention call
+ * followed by permute_attn_out (paroattention/cogvideox.py:216-227; wan.py:276,300): with
+ * out strides of a [B,N,H,D] buffer the result is token-major, ready for the output projection.
+ * Requires Nq == n_text + F*Hh*W.  orders: int32 [H] on the device. */
+int paro_attn_sparse_unpermute_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
+                                   const float* q_scale, const float* k_scale,
+                                   const float* v_scale, const float* v_mean,
+                                   const uint8_t* sparse, int64_t sparse_batch_stride,
+                                   void* out, int out_dtype, float* lse,
+                                   int B, int H, int Hkv, int Nq, int Nk, int D,
+                                   int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                                   int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                   int64_t o_stride_b, int64_t o_stride_h, int64_t o_stride_n,
+                                   float sm_scale, int is_causal, int flags,
+                                   const int32_t* orders, int n_text, int F, int Hh, int W,
+                                   void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * (2c) The reference's extension entry point in one call: V (fp16/bf16) -> FP8 tiles, then (2b).
  * Stands in for qk_int8_sv_f16_accum_f16_attn as bound at csrc/qattn/pybind_sm80.cpp:23 /

@@ -40,6 +40,10 @@ SIGNATURES = {
     "paro_attn_sparse_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _I, _P, _P,
                                      _I, _I, _I, _I, _I, _I,
                                      _L, _L, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I, _P]),
+    "paro_attn_sparse_unpermute_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _L, _P, _I, _P,
+                                               _I, _I, _I, _I, _I, _I,
+                                               _L, _L, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I,
+                                               _P, _I, _I, _I, _I, _P]),
     "paro_attn_workspace_bytes": (c_int64, [_I, _I, _I, _I]),
     "paro_qk_int8_sv_f16_attn": (c_int, [_P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _P, _P, _L,
                                          _I, _I, _I, _I, _I, _I,

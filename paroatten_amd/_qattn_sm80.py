@@ -121,7 +121,7 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
 
 
 def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_scale, sm_scale, sparse,
-                          is_causal=0, return_lse=0, exact_exp=False):
+                          is_causal=0, return_lse=0, exact_exp=False, unpermute=None):
     """The attention kernel alone, on operands that are already in its formats (HND, contiguous):
     q8/k8 int8 [B,H,N,D] / [B,Hkv,Nk,D], v8 = FP8 tiles from paro_v_fp8_pack or the fused
     preparation, v_scale / v_mean f32 [B,Hkv,D] (v_mean None: V was not mean-smoothed).  No
@@ -154,12 +154,24 @@ def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_
         _chk(tuple(sparse.shape) == (H, nbq, nbk), f"Tensor sparse must have shape ([{B},] {H}, {nbq}, {nbk})")
         sparse_bs = 0
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q8.device) if return_lse else torch.empty(0)
-    check(load().paro_attn_sparse_fwd(
-        ptr(q8), ptr(k8), ptr(v8), ptr(query_scale), ptr(key_scale), ptr(v_scale), ptr(v_mean), ptr(sparse), sparse_bs,
-        ptr(output), _lib.DTYPE_CODE[output.dtype], ptr(lse) if return_lse else None, None,
-        B, H, Hkv, Nq, Nk, D, q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
-        output.stride(0), output.stride(1), output.stride(2), float(sm_scale), int(is_causal),
-        _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0, stream_of(q8)))
+    flags = _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0
+    strides = (q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
+               output.stride(0), output.stride(1), output.stride(2))
+    if unpermute is None:
+        check(load().paro_attn_sparse_fwd(
+            ptr(q8), ptr(k8), ptr(v8), ptr(query_scale), ptr(key_scale), ptr(v_scale), ptr(v_mean), ptr(sparse),
+            sparse_bs, ptr(output), _lib.DTYPE_CODE[output.dtype], ptr(lse) if return_lse else None, None,
+            B, H, Hkv, Nq, Nk, D, *strides, float(sm_scale), int(is_causal), flags, stream_of(q8)))
+    else:
+        orders, grid, n_text = unpermute
+        _chk(orders.is_cuda and orders.dtype == torch.int32 and orders.dim() == 1 and orders.numel() == H
+             and orders.is_contiguous(), f"orders must be a contiguous int32 GPU tensor of {H} entries")
+        F_, Hh, W = (int(x) for x in grid)
+        check(load().paro_attn_sparse_unpermute_fwd(
+            ptr(q8), ptr(k8), ptr(v8), ptr(query_scale), ptr(key_scale), ptr(v_scale), ptr(v_mean), ptr(sparse),
+            sparse_bs, ptr(output), _lib.DTYPE_CODE[output.dtype], ptr(lse) if return_lse else None,
+            B, H, Hkv, Nq, Nk, D, *strides, float(sm_scale), int(is_causal), flags,
+            ptr(orders), int(n_text), F_, Hh, W, stream_of(q8)))
     return lse
 
 

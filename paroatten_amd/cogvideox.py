@@ -8,8 +8,8 @@ return value and `get_time_stats()`.  What changes underneath:
     are one pass that reads the projections in their native token-major memory ([B,N,H*D] viewed as
     [B,H,N,D] through strides) and writes only what the attention kernel reads: no transpose copy,
     no in-place rotate pass, no Python loop over heads, no host sync, no `.to(float16)` of V;
-  * the inverse permutation writes token-major memory directly, so the reshape for the output
-    projection is a view;
+  * the inverse permutation is folded into the attention kernel's stores, which go straight to
+    token-major memory, so the reshape for the output projection is a view;
   * (F,H,W), literals in the reference (cogvideox.py:31-33), are the `grid` argument/attribute;
   * timing is kept by events that are only read in get_time_stats(): no synchronize per call.
 """
@@ -124,12 +124,12 @@ class _ParoProcessorBase:
         km = PM.rope_k_mean(key, grid, n_text, cos, sin) if self.smooth_k else None
         return PM.rope_permute_quant(query, key, value, orders, grid, n_text, cos, sin, km=km)
 
-    def _sparse_attention(self, ops, dtype, sm_scale):
-        B, H, N, D = ops.q8.shape
-        out = torch.empty((B, H, N, D), dtype=dtype, device=ops.q8.device)
+    def _sparse_attention(self, ops, out, sm_scale, orders, grid, n_text):
+        """Block-sparse attention on the prepared operands; the inverse permutation (permute_attn_out)
+        is part of the kernel's stores, `out` is the [B,H,N,D] view of the token-major result."""
         qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, out, ops.q_scale, ops.k_scale,
-                                    sm_scale, self._mask(), exact_exp=self.exact_exp)
-        return out
+                                    sm_scale, self._mask(), exact_exp=self.exact_exp,
+                                    unpermute=(orders, grid, n_text))
 
     def get_time_stats(self):
         self._timer.fold(block=True)
@@ -192,9 +192,9 @@ class PARO_CogVideoXAttnProcessor2_0(_ParoProcessorBase):
             done.record()
         else:
             ops = self._prepare(query, key, value, orders, grid, text_seq_length, cos, sin, rotate_key)
-            out = self._sparse_attention(ops, query.dtype, 1.0 / (head_dim ** 0.5))
+            self._sparse_attention(ops, token_major.transpose(1, 2), 1.0 / (head_dim ** 0.5), orders, grid,
+                                   text_seq_length)
             done.record()
-            PM.permute_inverse(out, orders, grid, text_seq_length, out=token_major.transpose(1, 2))
         self.call_count += 1
         if len(self._timer._pending) >= 64:
             self._timer.fold(block=False)

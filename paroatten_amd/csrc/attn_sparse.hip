@@ -26,7 +26,7 @@
 // (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:44-726) as instantiated by its host (:1022-1048):
 // scale indexing :100-133, mask indexing :222/:268, out-of-range columns attn_utils.cuh:355-381,
 // softmax recurrence attn_utils.cuh:383-488, normalisation :786-840, lse = log2(d) + m (:711-723).
-#include "paro_common.hpp"
+#include "paro_device.hpp"
 #include <type_traits>
 
 namespace paro {
@@ -50,6 +50,10 @@ struct AttnParams {
   int B, H, Hkv, Nq, Nk, nbq, nbk;
   int total;  // B*H*nbq workgroups that have work
   float sm_scale_log2e;
+  // optional inverse permutation on the way out: q-row r of head h is stored at token
+  // n_text + unpermute(r - n_text, orders[h]) (rows below n_text stay); orders == nullptr: row r
+  const int* orders;
+  int n_text, F, Hh, W;
 };
 
 // P~ = 2^(S*c - m + P_EXP_OFFSET).  m is the running row maximum, refreshed lazily: only when a
@@ -213,10 +217,17 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
   const int cnt = s_cnt;
 
   using OutT = F16x<OUT_DT>;
-  unsigned short* outp = reinterpret_cast<unsigned short*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)qrow * p.os_n;
+  // where this lane's q-row goes (evaluated where it is needed: nothing of it lives across the loop)
+  auto out_row_ptr = [&]() {
+    int drow = qrow;
+    if (p.orders != nullptr && qrow >= p.n_text && qrow < p.Nq)
+      drow = p.n_text + unpermute_index(qrow - p.n_text, p.orders[h], p.F, p.Hh, p.W);
+    return reinterpret_cast<unsigned short*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)drow * p.os_n;
+  };
 
   if (cnt == 0) {  // no kept block: the row outputs 0 (reference: m = -5e6, d = 1, O = 0)
     if (qrow < p.Nq) {
+      unsigned short* outp = out_row_ptr();
 #pragma unroll
       for (int c = 0; c < D / 16; c++) *reinterpret_cast<v4i*>(outp + (lh * (D / 16) + c) * 8) = v4i{0, 0, 0, 0};
       if (p.lse && lh == 0) p.lse[((int64_t)b * p.H + h) * p.Nq + qrow] = -INFINITY;
@@ -582,6 +593,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
   const float d_tot = l32 < 16 ? d_lo : d_hi;
   const float inv = 1.0f / d_tot;
   if (qrow < p.Nq) {
+    unsigned short* outp = out_row_ptr();
     const float* vsc = p.v_scale + bhk * D;
     const float* vmn = p.v_mean ? p.v_mean + bhk * D : nullptr;
 #pragma unroll
@@ -638,14 +650,15 @@ static int dispatch_attn(const AttnParams& p, int is_causal, bool dump, bool exa
 
 }  // namespace paro
 
-extern "C" int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8, const float* q_scale,
-                                    const float* k_scale, const float* v_scale, const float* v_mean,
-                                    const uint8_t* sparse, int64_t sparse_batch_stride, void* out, int out_dtype,
-                                    float* lse, int32_t* s_dump, int B, int H, int Hkv, int Nq, int Nk, int D,
-                                    int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
-                                    int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
-                                    int64_t o_stride_n, float sm_scale, int is_causal, int flags, void* stream) {
-  using namespace paro;
+namespace paro {
+static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v8, const float* q_scale,
+                            const float* k_scale, const float* v_scale, const float* v_mean,
+                            const uint8_t* sparse, int64_t sparse_batch_stride, void* out, int out_dtype,
+                            float* lse, int32_t* s_dump, int B, int H, int Hkv, int Nq, int Nk, int D,
+                            int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
+                            int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
+                            int64_t o_stride_n, float sm_scale, int is_causal, int flags, const int32_t* orders,
+                            int n_text, int F, int Hh, int W, void* stream) {
   PARO_CHECK((flags & ~PARO_ATTN_EXACT_EXP) == 0, PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
   PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && v_scale && sparse && out, PARO_ERR_RUNTIME,
              "paro_attn_sparse_fwd: null tensor pointer");
@@ -676,6 +689,7 @@ extern "C" int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const ui
   p.B = B; p.H = H; p.Hkv = Hkv; p.Nq = Nq; p.Nk = Nk; p.nbq = nbq; p.nbk = nbk;
   p.total = B * H * nbq;
   p.sm_scale_log2e = sm_scale * 1.4426950408889634f;
+  p.orders = orders; p.n_text = n_text; p.F = F; p.Hh = Hh; p.W = W;
   hipStream_t st = (hipStream_t)stream;
   const bool dump = s_dump != nullptr;
   const bool exact = (flags & PARO_ATTN_EXACT_EXP) != 0;
@@ -685,6 +699,41 @@ extern "C" int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const ui
   }
   if (out_dtype == PARO_DTYPE_F16) return dispatch_attn<128, PARO_DTYPE_F16>(p, is_causal, dump, exact, st);
   return dispatch_attn<128, PARO_DTYPE_BF16>(p, is_causal, dump, exact, st);
+}
+}  // namespace paro
+
+extern "C" int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8, const float* q_scale,
+                                    const float* k_scale, const float* v_scale, const float* v_mean,
+                                    const uint8_t* sparse, int64_t sparse_batch_stride, void* out, int out_dtype,
+                                    float* lse, int32_t* s_dump, int B, int H, int Hkv, int Nq, int Nk, int D,
+                                    int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
+                                    int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
+                                    int64_t o_stride_n, float sm_scale, int is_causal, int flags, void* stream) {
+  return paro::attn_sparse_impl(q8, k8, v8, q_scale, k_scale, v_scale, v_mean, sparse, sparse_batch_stride, out,
+                                out_dtype, lse, s_dump, B, H, Hkv, Nq, Nk, D, q_stride_b, q_stride_h, q_stride_n,
+                                k_stride_b, k_stride_h, k_stride_n, o_stride_b, o_stride_h, o_stride_n, sm_scale,
+                                is_causal, flags, nullptr, 0, 0, 0, 0, stream);
+}
+
+extern "C" int paro_attn_sparse_unpermute_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
+                                              const float* q_scale, const float* k_scale, const float* v_scale,
+                                              const float* v_mean, const uint8_t* sparse,
+                                              int64_t sparse_batch_stride, void* out, int out_dtype, float* lse,
+                                              int B, int H, int Hkv, int Nq, int Nk, int D, int64_t q_stride_b,
+                                              int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
+                                              int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b,
+                                              int64_t o_stride_h, int64_t o_stride_n, float sm_scale, int is_causal,
+                                              int flags, const int32_t* orders, int n_text, int F, int Hh, int W,
+                                              void* stream) {
+  using namespace paro;
+  PARO_CHECK(orders, PARO_ERR_RUNTIME, "paro_attn_sparse_unpermute_fwd: null orders");
+  PARO_CHECK(n_text >= 0 && F > 0 && Hh > 0 && W > 0 && (int64_t)n_text + (int64_t)F * Hh * W == Nq, PARO_ERR_RUNTIME,
+             "paro_attn_sparse_unpermute_fwd: n_text + F*H*W = %d + %d*%d*%d does not equal the token count %d",
+             n_text, F, Hh, W, Nq);
+  return attn_sparse_impl(q8, k8, v8, q_scale, k_scale, v_scale, v_mean, sparse, sparse_batch_stride, out, out_dtype,
+                          lse, nullptr, B, H, Hkv, Nq, Nk, D, q_stride_b, q_stride_h, q_stride_n, k_stride_b,
+                          k_stride_h, k_stride_n, o_stride_b, o_stride_h, o_stride_n, sm_scale, is_causal, flags,
+                          orders, n_text, F, Hh, W, stream);
 }
 
 extern "C" int64_t paro_attn_workspace_bytes(int B, int Hkv, int Nk, int D) {

@@ -22,30 +22,6 @@
 
 namespace paro {
 
-// image index in permuted order -> image index in source (F,H,W row-major) order
-__device__ __forceinline__ int unpermute_index(int di, int order, int F, int Hh, int W) {
-  // axes in the permuted order, slowest first (cogvideox.py:38-45)
-  int s1, s2, a0, a1, a2;  // sizes of the two faster axes; which source axis each position is
-  switch (order) {
-    default:
-    case 0: a0 = 0; a1 = 1; a2 = 2; break;
-    case 1: a0 = 0; a1 = 2; a2 = 1; break;
-    case 2: a0 = 1; a1 = 2; a2 = 0; break;
-    case 3: a0 = 1; a1 = 0; a2 = 2; break;
-    case 4: a0 = 2; a1 = 1; a2 = 0; break;
-    case 5: a0 = 2; a1 = 0; a2 = 1; break;
-  }
-  const int S[3] = {F, Hh, W};
-  s1 = S[a1];
-  s2 = S[a2];
-  int c[3];
-  c[a2] = di % s2;
-  const int r = di / s2;
-  c[a1] = r % s1;
-  c[a0] = r / s1;
-  return (c[0] * Hh + c[1]) * W + c[2];
-}
-
 template <int DT, int D>
 __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
     const unsigned short* __restrict__ q_in, const unsigned short* __restrict__ k_in,

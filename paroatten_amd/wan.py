@@ -100,9 +100,8 @@ class PARO_WanAttnProcessor2_0(_ParoProcessorBase):
                                   device=query.device)
         if sparse:
             ops = self._prepare(query, key, value, orders, grid, 0, cos, sin)
-            out = self._sparse_attention(ops, query.dtype, 1.0 / (head_dim ** 0.5))
+            self._sparse_attention(ops, token_major.transpose(1, 2), 1.0 / (head_dim ** 0.5), orders, grid, 0)
             done.record()
-            PM.permute_inverse(out, orders, grid, 0, out=token_major.transpose(1, 2))
         else:
             qp, kp, vp = self._rope_permute(query, key, value, orders, grid, 0, cos, sin)
             out = F.scaled_dot_product_attention(qp, kp, vp, attn_mask=attention_mask, dropout_p=0.0, is_causal=False)

@@ -145,3 +145,32 @@ def test_fused_prep_rejects_bad_arguments(dev):
         PM.rope_permute_quant(q, q, q[:, :, :, :32], orders, (2, 8, 8), 0)
     with pytest.raises(RuntimeError):
         PM.rope_permute_quant(q, q, q, orders, (2, 8, 8), 0, km=torch.zeros(1, 2, 1, 64, device=dev))  # dtype
+
+
+@pytest.mark.parametrize("D,grid,n_text,dtype", [(64, (4, 6, 10), 16, torch.float16), (128, (3, 5, 9), 0, torch.bfloat16),
+                                                 (64, (3, 5, 7), 226, torch.bfloat16)])
+def test_attention_with_folded_inverse_permutation(dev, D, grid, n_text, dtype):
+    """paro_attn_sparse_unpermute_fwd == attention followed by the inverse permutation, bit for bit,
+    into a token-major buffer; an empty mask row still writes its zeros at the unpermuted places."""
+    from paroatten_amd import _qattn_sm80 as qattn
+    from paroatten_amd import permute as PM
+    B, H = 2, 5
+    N = n_text + grid[0] * grid[1] * grid[2]
+    q, k, v = (t.to(dev) for t in synth.make_qkv(B, H, N, D, dtype, seed=21))
+    plan = synth.make_permute_plan(1, H, seed=22)
+    orders = PM.head_orders(plan, 0, dev)
+    nb = (N + 63) // 64
+    mask = synth.make_block_mask(H, nb, 0.6, seed=23).to(dev)
+    mask[1, nb - 1, :] = False
+    ops = PM.rope_permute_quant(q, k, v, orders, grid, n_text)
+    plain = torch.empty((B, H, N, D), dtype=dtype, device=dev)
+    qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, plain, ops.q_scale, ops.k_scale,
+                                D ** -0.5, mask)
+    want = PM.permute_inverse(plain, orders, grid, n_text)
+    token_major = torch.full((B, N, H, D), 7.0, dtype=dtype, device=dev)
+    qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, token_major.transpose(1, 2),
+                                ops.q_scale, ops.k_scale, D ** -0.5, mask, unpermute=(orders, grid, n_text))
+    assert torch.equal(token_major.transpose(1, 2), want)
+    with pytest.raises(RuntimeError):
+        qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, plain, ops.q_scale, ops.k_scale,
+                                    D ** -0.5, mask, unpermute=(orders, (grid[0], grid[1], grid[2] + 1), n_text))
