@@ -1,23 +1,24 @@
 // Block-sparse quantised attention for gfx950 (MI355X).
 //
 //   S^T = K8 . Q8^T      v_mfma_i32_32x32x32_i8       exact int32
-//   P~  = 2^(S*c - m + 8) online base-2 softmax in fp32, rounded to FP8 e4m3 (OCP)
+//   P~  = 2^(S*c - m + 5) online base-2 softmax in fp32, rounded to FP8 e4m3 (OCP)
 //   O^T += V8^T . P~^T   v_mfma_f32_32x32x64_f8f6f4   fp32 accumulation
+//   d   += sum_j P~      v_mfma_f32_16x16x128_f8f6f4  against a selector operand
 //
 // One workgroup = one 64-row q-block of one (batch, head); its two 64-lane waves own 32 q-rows
 // each (= one q-scale group).  The transposed products make the accumulator fragment of S^T (a lane
 // holds 32 kv-values of ONE q-row) directly the B operand of the P.V MFMA; the kv-order inside a
 // block that this implies is absorbed by the tile order V8 is stored in (see v_fp8.hip), so no
-// cross-lane data movement is needed between the two matrix products and the row maximum / row sum
-// need one exchange with the partner lane (lane ^ 32) only.
+// cross-lane data movement is needed between the two matrix products and the row maximum needs one
+// exchange with the partner lane (lane ^ 32) only.
 //
 // k-blocks: the workgroup turns its row of the bool mask into a compact list in LDS and loops over
-// the kept blocks only; a skipped block costs neither loads nor MFMA issue.  K8 (row-major rows
-// padded by 16 bytes against bank conflicts) and V8 (already in fragment order) tiles go through a 3-stage
-// LDS ring, and the loop is software-pipelined: while the softmax of block i runs on the VALU, the
-// global loads of block i+2 are in flight, the K fragments of block i+1 and the V fragments of
-// block i are on their way out of LDS, and the iteration ends with Q.K^T of block i+1 issued ahead
-// of P.V of block i, so that the next softmax can start under the P.V MFMAs.  One barrier per block.
+// the kept blocks only; a skipped block costs neither loads nor MFMA issue.  K8 (row-major, 16-byte
+// chunks XOR-swizzled against bank conflicts) and V8 (already in fragment order) tiles come in by
+// LDS-DMA through a ring of three (D = 64) or two (D = 128) stages, and the loop is software-
+// pipelined: while the softmax weights of block i are computed on the VALU, the tiles of the next
+// blocks are in flight, and the MFMAs of P.V(i-1) and S^T(i+1) are issued one at a time from inside
+// the VALU stream.  One barrier per block.
 //
 // Workgroups are renumbered so that each of the 8 XCDs walks a contiguous range of (batch, head,
 // q-block): the K8/V8 of the one or two heads an XCD is working on stay resident in its own L2.

@@ -120,3 +120,39 @@ def test_mask_generator_contract():
     assert torch.equal(synth.make_block_mask(2, 16, 0.4, seed=5), synth.make_block_mask(2, 16, 0.4, seed=5))
     plan = synth.make_permute_plan(4, 48, seed=0)
     assert plan["permute"].shape == (4, 48) and int(plan["permute"].min()) >= 0 and int(plan["permute"].max()) <= 5
+
+
+def test_new_entry_points_validate_without_gpu():
+    """the one-pass preparation, the folded inverse permutation and the mask bit kernels reject bad
+    arguments before any launch"""
+    import paroatten_amd._lib as L
+    lib = L.load()
+    assert lib.paro_mask_bits_bytes(0) == 0 and lib.paro_mask_bits_bytes(9) == 2 and lib.paro_mask_bits_bytes(-3) == 0
+    assert lib.paro_mask_pack(None, None, 0, None) == L.PARO_OK            # nothing to do
+    assert lib.paro_mask_pack(None, None, 16, None) == L.PARO_ERR_RUNTIME and b"null" in lib.paro_last_error()
+    assert lib.paro_mask_unpack(None, None, -1, None) == L.PARO_ERR_INVALID_VALUE
+    buf = ctypes.create_string_buffer(8192)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 255) & ~255)
+    odd = ctypes.c_void_p(p.value + 4)
+    assert lib.paro_mask_unpack(odd, p, 64, None) == L.PARO_ERR_RUNTIME and b"aligned" in lib.paro_last_error()
+    assert lib.paro_prep_workspace_bytes(2, 48, 17776, 64) == 2 * 48 * 70 * 3 * 64 * 4
+
+    def prep(D=64, N=128, grid=(2, 8, 8), n_text=0, q=p, ws=p, ws_bytes=1 << 20):
+        return lib.paro_rope_permute_quant_fwd(q, p, p, 0, None, None, p, None, p, p, p, p, p, p, p, ws, ws_bytes,
+                                               1, 1, N, D, n_text, grid[0], grid[1], grid[2],
+                                               N * D, N * D, D, N * D, N * D, D, N * D, N * D, D, 0, 0, 1, None)
+    assert prep(D=96) == L.PARO_ERR_INVALID_VALUE and lib.paro_last_error() == b"Unsupported head dim: 96"
+    assert prep(grid=(2, 8, 9)) == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
+    assert prep(q=None) == L.PARO_ERR_RUNTIME and b"null" in lib.paro_last_error()
+    assert prep(ws_bytes=16) == L.PARO_ERR_RUNTIME and b"workspace" in lib.paro_last_error()
+
+    rc = lib.paro_attn_sparse_unpermute_fwd(p, p, p, p, p, p, p, p, 0, p, 0, None, 1, 1, 1, 128, 128, 64,
+                                            8192, 8192, 64, 8192, 8192, 64, 8192, 8192, 64, 0.125, 0, 0,
+                                            None, 0, 2, 8, 8, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"null orders" in lib.paro_last_error()
+    rc = lib.paro_attn_sparse_unpermute_fwd(p, p, p, p, p, p, p, p, 0, p, 0, None, 1, 1, 1, 128, 128, 64,
+                                            8192, 8192, 64, 8192, 8192, 64, 8192, 8192, 64, 0.125, 0, 0,
+                                            p, 1, 2, 8, 8, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
+    rc = lib.paro_rope_k_mean(p, 0, p, None, p, p, 1 << 20, 1, 1, 128, 64, 0, 2, 8, 8, 8192, 8192, 64, 64, 64, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"cos and sin" in lib.paro_last_error()
