@@ -53,7 +53,6 @@ __global__ void __launch_bounds__(256) rope_permute_kernel(
   }
   const int bh0 = blockIdx.y * heads_per_wg;
   const int bh1 = min(BH, bh0 + heads_per_wg);
-#pragma unroll 2
   for (int bh = bh0; bh < bh1; bh++) {
     const int b = bh / H, head = bh - b * H;
     int mapped = tok;

@@ -166,3 +166,26 @@ def test_int32_qk_accumulators_bitexact(dev, D):
     assert (dump[~keep] == -(2 ** 31)).all()
     # (rows/columns past N inside computed blocks hold products with a re-read last row; the
     # kernel masks those columns out of the softmax and never stores those rows)
+
+
+def test_nhd_layout_and_paroattn_entry(dev):
+    """tensor_layout="NHD" ([B,N,H,D]) gives exactly the HND result; `paroattn` with sparse=None is the
+    all-true mask (core.py:13-85 of the reference documents both and can run neither)."""
+    import paroatten_amd as P
+    B, H, N, D = 2, 3, 700, 64
+    q, k, v = synth.make_qkv(B, H, N, D, torch.float16, seed=31)
+    nb = (N + 63) // 64
+    mask = synth.make_block_mask(H, nb, 0.5, seed=32).to(dev)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    o_hnd, lse_hnd = P.paroattn_qk_int8_pv_fp16_cuda(qd, kd, vd, mask, return_lse=True)
+    qn, kn, vn = (t.transpose(1, 2).contiguous() for t in (qd, kd, vd))
+    o_nhd, lse_nhd = P.paroattn_qk_int8_pv_fp16_cuda(qn, kn, vn, mask, tensor_layout="NHD", return_lse=True)
+    assert o_nhd.shape == (B, N, H, D)
+    assert torch.equal(o_nhd.transpose(1, 2), o_hnd) and torch.equal(lse_nhd, lse_hnd)
+    dense = P.paroattn(qd, kd, vd, smooth_k=True)
+    full = P.paroattn_qk_int8_pv_fp16_cuda(qd, kd, vd, torch.ones(H, nb, nb, dtype=torch.bool, device=dev),
+                                           smooth_k=True)
+    assert torch.equal(dense, full)
+    # against attention on the UNQUANTISED tensors: INT8 Q/K (K smoothed) and FP8 P/V together
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    assert cosine(dense.cpu(), ref) >= 0.998
