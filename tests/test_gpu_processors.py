@@ -216,3 +216,56 @@ def test_processor_rejects_unknown_grid(dev):
     proc.sparse_mask = masks.to(dev)
     with pytest.raises(ValueError):
         proc(attn, hidden, text)
+
+
+@torch.no_grad()
+def test_pipeline_wiring_over_layers_and_steps(dev):
+    """set_paro_processors + TimestepCallback on a stand-in transformer: three blocks, five denoising
+    steps mapped onto two mask timesteps; the prefetch-stream run equals the resident-mask run in every
+    block and step, and the mask timestep follows the callback's arithmetic."""
+    import types
+
+    from paroatten_amd import wan
+    from paroatten_amd.prefetch_utils import SparseMaskPrefetchStream, TimestepCallback, mask_timestep_index
+    H, D, grid, n_text, B, L, T, steps = 2, 64, (2, 4, 8), 0, 1, 3, 2, 5
+    N = grid[0] * grid[1] * grid[2]
+    nb = (N + 63) // 64
+    masks = torch.stack([torch.stack([synth.make_block_mask(H, nb, 0.7, seed=50 + t * L + l, band=0) for l in range(L)])
+                         for t in range(T)])
+    plan = synth.make_permute_plan(L, H, seed=51)
+
+    def make_transformer():
+        blocks = [types.SimpleNamespace(attn1=_Attn(H, D, "rms", seed=60 + i).to(dev, torch.bfloat16)) for i in range(L)]
+        for b in blocks:
+            b.attn1.processor = None
+        return types.SimpleNamespace(blocks=blocks)
+
+    ta, tb = make_transformer(), make_transformer()
+    pa = wan.set_paro_processors(ta, plan, sparse_mask=masks.to(dev), grid=grid)
+    stream = SparseMaskPrefetchStream(masks, device=dev)
+    pb = wan.set_paro_processors(tb, plan, prefetch_stream=stream, grid=grid)
+    assert [p.i_block for p in pa] == [0, 1, 2] and all(p.i_timestep == 0 for p in pb)
+    assert all(isinstance(p, wan.PARO_WanAttnProcessor2_0) for p in pa)
+    with pytest.raises(ValueError):
+        wan.set_paro_processors(ta, plan)
+    cb_a, cb_b = TimestepCallback(T), TimestepCallback(T)
+    sched = types.SimpleNamespace(timesteps=list(range(steps)))
+    pipe_a = types.SimpleNamespace(transformer=ta, scheduler=sched)
+    pipe_b = types.SimpleNamespace(transformer=tb, scheduler=sched)
+    g = torch.Generator().manual_seed(52)
+    x = torch.randn(B, N, H * D, generator=g).to(dev, torch.bfloat16)
+    freqs = O.rope_table_wan(D, grid).to(dev)
+    seen = []
+    for step in range(steps):
+        ha = hb = x
+        for l in range(L):
+            ha = ta.blocks[l].attn1.processor(ta.blocks[l].attn1, ha, rotary_emb=freqs)
+            hb = tb.blocks[l].attn1.processor(tb.blocks[l].attn1, hb, rotary_emb=freqs)
+            assert torch.equal(ha, hb), (step, l)
+        seen.append(pa[0].i_timestep)
+        cb_a.on_step_end(pipe_a, step, torch.tensor(float(step)), {})
+        cb_b.on_step_end(pipe_b, step, torch.tensor(float(step)), {})
+    want = [0] + [min(mask_timestep_index(s, steps, T), T) for s in range(steps - 1)]
+    assert seen == want and ta.i_timestep == mask_timestep_index(steps - 1, steps, T)
+    assert stream.i_iter == steps * L
+    assert sum(p.call_count for p in pb) == steps * L and pb[0].get_time_stats()["total_ms"] > 0
