@@ -113,8 +113,8 @@ static int launch_rp(const void* q_in, const void* k_in, const void* v_in, void*
   const int BH = B * H;
   // enough (batch, head) pairs per workgroup to amortise the rotary fragment, few enough that the
   // launch still has several thousand workgroups
-  int hpw = 8;
-  while (hpw > 1 && (int64_t)ceil_div(N, rows) * ceil_div(BH, hpw) < 4096) hpw >>= 1;
+  int hpw = 16;
+  while (hpw > 1 && (int64_t)ceil_div(N, rows) * ceil_div(BH, hpw) < 3072) hpw >>= 1;
   dim3 grid(ceil_div(N, rows), ceil_div(BH, hpw)), block(256);
 #define PARO_RP(DTV, DV)                                                                                          \
   hipLaunchKernelGGL((rope_permute_kernel<DTV, DV, INVERSE>), grid, block, 0, st, (const unsigned short*)q_in,    \
