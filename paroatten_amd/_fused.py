@@ -62,11 +62,11 @@ def _quant(input, mean, output, scale, group, n_groups_fn, tensor_layout, sm_sca
     if mean is not None:
         _chk(tuple(mean.shape) == (B, H, D), "Tensor mean must have shape (batch_size, num_heads, head_dim)")
     ms_b, ms_h = (mean.stride(0), mean.stride(1)) if mean is not None else (0, 0)
-    check(load().paro_quant_int8(
+    _lib.on(input).paro_quant_int8(
         ptr(input), _lib.DTYPE_CODE[input.dtype], ptr(mean), ptr(output), ptr(scale),
         B, H, N, D, input.stride(0), xs_h, xs_n, ms_b, ms_h, output.stride(0), os_h, os_n,
         scale.stride(0), scale.stride(1), group, n_groups,
-        0 if sm_scale is None else 1, 0.0 if sm_scale is None else float(sm_scale), stream_of(input)))
+        0 if sm_scale is None else 1, 0.0 if sm_scale is None else float(sm_scale), stream_of(input))
 
 
 def _block_groups(block_size):
@@ -127,9 +127,9 @@ def sub_mean_cuda(input, mean, output, tensor_layout):
     _chk(tuple(mean.shape) == (B, H, D), "Tensor mean must have shape (batch_size, num_heads, head_dim)")
     _chk(tuple(output.shape) == tuple(input.shape),
          "Tensor output must have shape (input.size(0), input.size(1), input.size(2), input.size(3))")
-    check(load().paro_sub_mean(ptr(input), _lib.DTYPE_CODE[input.dtype], ptr(mean), ptr(output), B, H, N, D,
+    _lib.on(input).paro_sub_mean(ptr(input), _lib.DTYPE_CODE[input.dtype], ptr(mean), ptr(output), B, H, N, D,
                                input.stride(0), vs_h, vs_n, mean.stride(0), mean.stride(1),
-                               output.stride(0), os_h, os_n, stream_of(input)))
+                               output.stride(0), os_h, os_n, stream_of(input))
 
 
 _NV_LAYOUT = (

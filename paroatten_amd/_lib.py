@@ -112,3 +112,24 @@ def require_gpu(t: torch.Tensor, name: str):
     # same wording as CHECK_CUDA of the reference (csrc/utils.cuh:20-21)
     if not t.is_cuda:
         raise RuntimeError(f"Tensor {name} must be a CUDA tensor")
+
+
+class _OnDevice:
+    """`on(t).paro_xxx(args)`: the C ABI launches on the CURRENT device, so the call runs under a
+    device guard for the tensor's device (the reference works around the missing guard with
+    torch.cuda.set_device, paroattention/core.py:168-174) and its return code goes through check()."""
+
+    def __init__(self, t):
+        self._device = t.device
+
+    def __getattr__(self, name):
+        fn = getattr(load(), name)
+
+        def call(*args):
+            with torch.cuda.device(self._device):
+                check(fn(*args))
+        return call
+
+
+def on(t: torch.Tensor) -> _OnDevice:
+    return _OnDevice(t)

@@ -106,7 +106,7 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
     else:
         _chk(workspace.is_cuda and workspace.is_contiguous() and workspace.numel() * workspace.element_size() >= need,
              f"workspace must be a contiguous GPU buffer of at least {need} bytes")
-    check(load().paro_qk_int8_sv_f16_attn(
+    _lib.on(query).paro_qk_int8_sv_f16_attn(
         ptr(query), ptr(key), ptr(value), _lib.DTYPE_CODE[value.dtype], ptr(output), _lib.DTYPE_CODE[output.dtype],
         ptr(query_scale), ptr(key_scale), ptr(sparse), sparse_bs, ptr(lse) if return_lse else None,
         ptr(workspace), workspace.numel() * workspace.element_size(),
@@ -116,7 +116,7 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
         value.stride(0), value.stride(sh), value.stride(sn),
         output.stride(0), output.stride(sh), output.stride(sn),
         tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0,
-        _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0, stream_of(query)))
+        _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0, stream_of(query))
     return lse
 
 
@@ -158,20 +158,20 @@ def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_
     strides = (q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
                output.stride(0), output.stride(1), output.stride(2))
     if unpermute is None:
-        check(load().paro_attn_sparse_fwd(
+        _lib.on(q8).paro_attn_sparse_fwd(
             ptr(q8), ptr(k8), ptr(v8), ptr(query_scale), ptr(key_scale), ptr(v_scale), ptr(v_mean), ptr(sparse),
             sparse_bs, ptr(output), _lib.DTYPE_CODE[output.dtype], ptr(lse) if return_lse else None, None,
-            B, H, Hkv, Nq, Nk, D, *strides, float(sm_scale), int(is_causal), flags, stream_of(q8)))
+            B, H, Hkv, Nq, Nk, D, *strides, float(sm_scale), int(is_causal), flags, stream_of(q8))
     else:
         orders, grid, n_text = unpermute
         _chk(orders.is_cuda and orders.dtype == torch.int32 and orders.dim() == 1 and orders.numel() == H
              and orders.is_contiguous(), f"orders must be a contiguous int32 GPU tensor of {H} entries")
         F_, Hh, W = (int(x) for x in grid)
-        check(load().paro_attn_sparse_unpermute_fwd(
+        _lib.on(q8).paro_attn_sparse_unpermute_fwd(
             ptr(q8), ptr(k8), ptr(v8), ptr(query_scale), ptr(key_scale), ptr(v_scale), ptr(v_mean), ptr(sparse),
             sparse_bs, ptr(output), _lib.DTYPE_CODE[output.dtype], ptr(lse) if return_lse else None,
             B, H, Hkv, Nq, Nk, D, *strides, float(sm_scale), int(is_causal), flags,
-            ptr(orders), int(n_text), F_, Hh, W, stream_of(q8)))
+            ptr(orders), int(n_text), F_, Hh, W, stream_of(q8))
     return lse
 
 

@@ -36,7 +36,7 @@ def rope_permutation(Q: torch.Tensor, K: torch.Tensor, freq: torch.Tensor, permu
     QO = torch.empty((bs, n, dim), dtype=torch.float16, device=Q.device)
     KO = torch.empty((bs, n, dim), dtype=torch.float16, device=Q.device)
     # [bs, n, heads, 128] seen as (batch, head, token, channel) through strides
-    check(load().paro_rope_permute_fwd(
+    _lib.on(Q).paro_rope_permute_fwd(
         ptr(Q), ptr(K), None, ptr(QO), ptr(KO), None, _lib.DTYPE_CODE[torch.float16], ptr(cos), ptr(sin),
-        ptr(orders), bs, heads, n, 128, 0, 1, H, W, n * dim, 128, dim, n * dim, 128, dim, stream_of(Q)))
+        ptr(orders), bs, heads, n, 128, 0, 1, H, W, n * dim, 128, dim, n * dim, 128, dim, stream_of(Q))
     return QO, KO

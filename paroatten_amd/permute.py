@@ -67,11 +67,11 @@ def rope_permute(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Option
                 raise RuntimeError(f"Tensor {n} must be contiguous float32 of shape ({F * Hh * W}, {D})")
     outs = [None if t is None else torch.empty((B, H, N, D), dtype=t.dtype, device=t.device) for t in (q, k, v)]
     o_ref = next(o for o in outs if o is not None)
-    check(load().paro_rope_permute_fwd(
+    _lib.on(ref).paro_rope_permute_fwd(
         ptr(q), ptr(k), ptr(v), ptr(outs[0]), ptr(outs[1]), ptr(outs[2]), _lib.DTYPE_CODE[ref.dtype],
         ptr(cos), ptr(sin), ptr(orders), B, H, N, D, int(n_text), F, Hh, W,
         ref.stride(0), ref.stride(1), ref.stride(2), o_ref.stride(0), o_ref.stride(1), o_ref.stride(2),
-        stream_of(ref)))
+        stream_of(ref))
     return tuple(outs)
 
 
@@ -106,9 +106,9 @@ def rope_k_mean(k: torch.Tensor, grid: Sequence[int], n_text: int, cos: Optional
     lib = load()
     km = torch.empty((B, H, 1, D), dtype=k.dtype, device=k.device)
     ws = torch.empty(int(lib.paro_prep_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=k.device)
-    check(lib.paro_rope_k_mean(ptr(k), _lib.DTYPE_CODE[k.dtype], ptr(cos), ptr(sin), ptr(km), ptr(ws), ws.numel(),
+    _lib.on(k).paro_rope_k_mean(ptr(k), _lib.DTYPE_CODE[k.dtype], ptr(cos), ptr(sin), ptr(km), ptr(ws), ws.numel(),
                                B, H, N, D, int(n_text), F, Hh, W, k.stride(0), k.stride(1), k.stride(2),
-                               km.stride(0), km.stride(1), stream_of(k)))
+                               km.stride(0), km.stride(1), stream_of(k))
     return km
 
 
@@ -146,11 +146,11 @@ def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders
     v_scale = torch.empty((B, H, D), dtype=torch.float32, device=dev)
     v_mean = torch.empty((B, H, D), dtype=torch.float32, device=dev)
     ws = torch.empty(int(lib.paro_prep_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=dev)
-    check(lib.paro_rope_permute_quant_fwd(
+    _lib.on(q).paro_rope_permute_quant_fwd(
         ptr(q), ptr(k), ptr(v), _lib.DTYPE_CODE[q.dtype], ptr(cos), ptr(sin), ptr(orders), ptr(km),
         ptr(q8), ptr(q_scale), ptr(k8), ptr(k_scale), ptr(v8), ptr(v_scale), ptr(v_mean), ptr(ws), ws.numel(),
         B, H, N, D, int(n_text), F, Hh, W, q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1),
-        k.stride(2), v.stride(0), v.stride(1), v.stride(2), ms_b, ms_h, 1 if smooth_v else 0, stream_of(q)))
+        k.stride(2), v.stride(0), v.stride(1), v.stride(2), ms_b, ms_h, 1 if smooth_v else 0, stream_of(q))
     return PreparedOperands(q8, q_scale, k8, k_scale, v8, v_scale, v_mean if smooth_v else None)
 
 
@@ -170,9 +170,9 @@ def permute_inverse(o: torch.Tensor, orders: torch.Tensor, grid: Sequence[int], 
         _check_hnd(out, "out")
         if out.shape != o.shape or out.dtype != o.dtype or out.device != o.device:
             raise RuntimeError("out must have attn_out's shape, dtype and device")
-    check(load().paro_permute_inv(ptr(o), ptr(out), _lib.DTYPE_CODE[o.dtype], ptr(orders), B, H, N, D, int(n_text),
+    _lib.on(o).paro_permute_inv(ptr(o), ptr(out), _lib.DTYPE_CODE[o.dtype], ptr(orders), B, H, N, D, int(n_text),
                                   F, Hh, W, o.stride(0), o.stride(1), o.stride(2),
-                                  out.stride(0), out.stride(1), out.stride(2), stream_of(o)))
+                                  out.stride(0), out.stride(1), out.stride(2), stream_of(o))
     return out
 
 
@@ -181,7 +181,7 @@ def permute_index_map(orders: torch.Tensor, grid: Sequence[int]) -> torch.Tensor
     _check_orders(orders, orders.numel())
     F, Hh, W = (int(x) for x in grid)
     idx = torch.empty((orders.numel(), F * Hh * W), dtype=torch.int32, device=orders.device)
-    check(load().paro_permute_index_map(ptr(idx), ptr(orders), orders.numel(), F, Hh, W, stream_of(idx)))
+    _lib.on(idx).paro_permute_index_map(ptr(idx), ptr(orders), orders.numel(), F, Hh, W, stream_of(idx))
     return idx
 
 

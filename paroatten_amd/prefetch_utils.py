@@ -125,8 +125,8 @@ class SparseMaskPrefetchStream:
             if after is not None:
                 self.stream.wait_event(after)
             self._bits[buf].copy_(self.sparse_mask[index], non_blocking=True)
-            check(load().paro_mask_unpack(ptr(self._bits[buf]), ptr(self.double_buffer[buf]), self.mask_elems,
-                                          _lib.stream_of(self._bits[buf])))
+            _lib.on(self._bits[buf]).paro_mask_unpack(ptr(self._bits[buf]), ptr(self.double_buffer[buf]), self.mask_elems,
+                                          _lib.stream_of(self._bits[buf]))
             self._ready[buf].record(self.stream)
         self._held[buf] = index
 

@@ -101,7 +101,7 @@ def per_channel_fp8(v: torch.Tensor, tensor_layout: str = "HND", scale_max: floa
     vm = torch.empty((b, h, d), dtype=torch.float32, device=v.device)
     partial = torch.empty(int(lib.paro_v_fp8_partial_floats(b, h, n, d)), dtype=torch.float32, device=v.device)
     sn, sh = (2, 1) if tensor_layout == "HND" else (1, 2)
-    check(lib.paro_v_fp8_pack(ptr(v), _lib.DTYPE_CODE[v.dtype], ptr(v_fp8), ptr(v_scale), ptr(vm), ptr(partial),
+    _lib.on(v).paro_v_fp8_pack(ptr(v), _lib.DTYPE_CODE[v.dtype], ptr(v_fp8), ptr(v_scale), ptr(vm), ptr(partial),
                               b, h, n, d, v.stride(0), v.stride(sh), v.stride(sn), 1 if smooth_v else 0,
-                              stream_of(v)))
+                              stream_of(v))
     return v_fp8, v_scale, (vm if smooth_v else None)
