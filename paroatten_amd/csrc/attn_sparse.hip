@@ -334,6 +334,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
   v8i ones = {sel_word, sel_word, sel_word, sel_word, sel_word, sel_word, sel_word, sel_word};
   asm volatile("" : "+v"(ones));  // same: resident constant operand
   float m_i = -1e30f;
+  float m_thr = -1e30f, m_off = 0.f, m_off8 = 0.f;  // m + headroom and the m-dependent offsets (see step)
   float d_exact = 0.f;  // LSE only: sum of the unrounded P~ of this lane's 32 kv-columns per block
 
   // ---- prologue ------------------------------------------------------------------------------
@@ -408,6 +409,12 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     const int kidx_v = (int)klist[it + 4];
     read_v_frags(svp);
     const float c_next = qsc * clist[it + 1];
+    // scale of this block and what follows from it and from the current maximum alone
+    const float c = c_cur;
+    const float nmc = -S_MAGIC_F * c;
+    const float c8 = (8.0f / 65535.0f) * c;
+    float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
+    float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: byte = (8*(t + 7) + shift) / 65535
 
     // -- row maximum of this block
     float s[2][16];
@@ -443,19 +450,25 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     mx2 = max3(mx2, s[1][7], s[1][15]);
     float smax = max3(mx0, mx1, mx2);
     smax = max3(smax, mx3, mx3);
-    smax = partner_max(smax) - S_MAGIC_F;  // exact: both are integers below 2^24
+    smax = partner_max(smax);  // still biased by 1.5*2^23
 
-    const float c = c_cur;
-    const float m_blk = smax * c;
     // Lazy refresh of the running maximum (rare after the first few blocks).  The new maximum
     // applies to this block's weights at once; O and the row sums, which the pending P.V of the
     // previous block still has to reach through the stream below, are rescaled after the stream.
-    const bool refresh = __ballot(m_blk > m_i + P_HEADROOM) != 0ull;
+    // Everything that depends on m only (threshold, offsets of the affine maps) is state that changes
+    // on a refresh, so the common path goes from the maximum straight to the comparison.
+    const float m_blk = fmaf(smax, c, nmc);
+    const bool refresh = __ballot(m_blk > m_thr) != 0ull;
     float alpha = 1.0f;
     if (refresh) {
       const float m_new = fmaxf(m_i, m_blk);
       alpha = __builtin_amdgcn_exp2f(m_i - m_new);
       m_i = m_new;
+      m_thr = m_new + P_HEADROOM;
+      m_off = P_EXP_OFFSET - m_new;
+      m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT) * (1.0f / 65535.0f);
+      bias = fmaf(-S_MAGIC_F, c, m_off);
+      bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
       if constexpr (LSE) d_exact *= alpha;
     }
 
@@ -463,9 +476,6 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     //    after each chunk one MFMA goes to the matrix pipe: first S^T of the NEXT block, then the
     //    pending P.V of the PREVIOUS block.  All their operands are ready before the stream starts.
     float rs = 0.f;
-    const float bias = fmaf(-S_MAGIC_F, c, P_EXP_OFFSET - m_i);
-    const float c8 = (8.0f / 65535.0f) * c;
-    const float bias8 = fmaf(-S_MAGIC_F, c8, (8.0f * (P_EXP_OFFSET + 7.0f - m_i) + FAST_EXP_SHIFT) * (1.0f / 65535.0f));
     // MFMA issue plan: the pending P.V first (its operands are ready), S^T row tile 0 of the next
     // block once chunk 3 has read the last of the current one, row tile 1 after chunk 7
     // The K fragments of the next block (k-step r, both row tiles) are fetched from LDS right after
@@ -575,7 +585,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     // stage i-1 and writes V stage i+1
     int i3 = 0;  // it % 3
     for (int it = 0; it < cnt; it += 2) {
-      const int s1 = i3 == 2 ? 0 : i3 + 1, s2 = i3 == 0 ? 2 : i3 - 1;  // (i3+1)%3, (i3+2)%3 == (i3-1)%3
+      const int s1 = i3 == 2 ? 0 : i3 + 1, s2 = 3 - i3 - s1;  // (i3+1)%3 and the remaining stage (i3+2)%3
       step(it, i3, s1, s2, s1, pf_a, pf_b);
       if (it + 1 >= cnt) { i3 = s1; break; }
       step(it + 1, s1, s2, i3, s2, pf_b, pf_a);
