@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-Workload: BASELINE config 2, the CogVideoX-5b self-attention shape (B=2 CFG, H=48, D=64, fp16,
+Workload: benchmark configuration 2, the CogVideoX-5b self-attention shape (B=2 CFG, H=48, D=64, fp16,
 N=17776 tokens = 278 blocks of 64), seeded synthetic Q/K/V with a per-channel bias on K, per-head
 banded-plus-random 64x64 block masks.  One step = one call of the reference's extension entry point
 `qk_int8_sv_f16_accum_f16_attn` (what the reference's own bench/bench.py times) at density 0.3:

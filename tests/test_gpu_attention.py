@@ -37,9 +37,9 @@ def _run(dev, B, H, N, D, dtype, density, seed, Hkv=None, causal=False, smooth_k
 
 
 def _assert_close(o, o_ref, baseline_shape=False):
-    """atol 2e-2 and cosine >= 0.999 at the BASELINE shapes.  The FP8 P.V error is relative
+    """atol 2e-2 and cosine >= 0.999 at the benchmark shapes.  The FP8 P.V error is relative
     (about 3.5 % RMS of the output magnitude, measured), so on the reduced shapes below, whose
-    short rows give outputs several times larger than any BASELINE shape does, the absolute bound
+    short rows give outputs several times larger than any benchmark shape does, the absolute bound
     scales with the largest output instead: 8 % of max|o_ref| (never below 2e-2)."""
     err = (o.float() - o_ref.float()).abs().max().item()
     c = cosine(o, o_ref)
@@ -49,7 +49,7 @@ def _assert_close(o, o_ref, baseline_shape=False):
 
 
 def test_cfg0_plumbing(dev):
-    """BASELINE config 0: B=1,H=2,D=64,fp16,N=4096, density 0.5, K bias.  With lse the kernel
+    """benchmark configuration 0: B=1,H=2,D=64,fp16,N=4096, density 0.5, K bias.  With lse the kernel
     evaluates exact exponentials; without, its default fast path builds the e4m3 weights directly."""
     o, lse, o_ref, lse_ref, _ = _run(dev, 1, 2, 4096, 64, torch.float16, 0.5, seed=0)
     _assert_close(o, o_ref, baseline_shape=True)

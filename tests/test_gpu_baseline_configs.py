@@ -1,4 +1,4 @@
-"""GPU parity at the BASELINE shapes.  The kernels run on the full (B, H) extent where the memory of
+"""GPU parity at the benchmark shapes.  The kernels run on the full (B, H) extent where the memory of
 the test is bounded, the oracle checks whole heads of it (every head is independent), and
 size-independent properties cover the rest: permutation round trips, bit-exact re-quantisation,
 all-true masks against dense attention, zero rows for empty mask rows."""
@@ -25,7 +25,7 @@ def _check_heads(dev, wl, density, heads, seed, n_heads_total=None, with_rope=Fa
     """Run the path (permute [+ RoPE] -> quant (K smoothed) -> sparse attention -> inverse permute)
     on `n_heads_total` heads of workload `wl` and compare the listed heads with the oracle.
 
-    Without RoPE (what BASELINE configs 2-4 describe: N(0,1) Q/K/V, a per-channel bias on K that the
+    Without RoPE (what benchmark configurations 2-4 describe: N(0,1) Q/K/V, a per-channel bias on K that the
     mean smoothing removes) attention is diffuse and the bar is atol 2e-2 / cosine 0.999 on every
     element.  With RoPE the rotated K bias makes rows that one to three tokens dominate; there the
     absolute error is FP8's relative rounding error times an output of order 0.5, so the elementwise
