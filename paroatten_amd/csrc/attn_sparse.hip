@@ -81,11 +81,27 @@ __device__ __forceinline__ void cvt_pk_fp8(int& w, float a, float b) {
   else asm("v_cvt_pk_fp8_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));  // upper half: don't care, overwritten next
 }
 
-// two floats in [0,1] -> round(x * 65535) as two unsigned 16-bit fields (negative inputs give 0)
-__device__ __forceinline__ int cvt_pknorm_u16(float a, float b) {
+// a*b + c clamped to [0,1] (the clamp is an output modifier: no extra instruction)
+__device__ __forceinline__ float fma_clamp01(float a, float b, float c) {
+  float r;
+  asm("v_fma_f32 %0, %1, %2, %3 clamp" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// two floats in [0,1] -> round(x * 32767) as two 16-bit fields (never negative, at most 0x7FFF)
+__device__ __forceinline__ int cvt_pknorm_i16(float a, float b) {
   int w;
-  asm("v_cvt_pknorm_u16_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));
+  asm("v_cvt_pknorm_i16_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));
   return w;
+}
+
+// field-wise maximum of three words of two non-negative 16-bit integers each: on such bit patterns
+// (small ones are half-precision denormals, 0x7C01.. are NaNs, which propagate) the packed
+// half-precision maximum orders like the integers, and a NaN still reads as "large"
+__device__ __forceinline__ int pk_max3_fields(int a, int b, int c) {
+  int r;
+  asm("v_pk_maximum3_f16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
 }
 
 __device__ __forceinline__ int lshl8_or(int hi, int lo) {
@@ -412,9 +428,9 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
     // scale of this block and what follows from it and from the current maximum alone
     const float c = c_cur;
     const float nmc = -S_MAGIC_F * c;
-    const float c8 = (8.0f / 65535.0f) * c;
+    const float c8 = (8.0f / 32767.0f) * c;
     float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
-    float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: byte = (8*(t + 7) + shift) / 65535
+    float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: byte = (8*(t + 7) + shift) / 32767
 
     // -- row maximum of this block
     float s[2][16];
@@ -436,40 +452,48 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
         }
     }
 
-    // four interleaved v_max3 chains (the values are integers read as floats: no NaN to canonicalise)
-    float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[0][8], s[0][9], s[0][10]);
-    float mx2 = max3(s[1][0], s[1][1], s[1][2]), mx3 = max3(s[1][8], s[1][9], s[1][10]);
+    // Row maximum of the block (biased by 1.5*2^23 like the scores), as the log2-domain score m_blk
+    auto block_max = [&]() {
+      // four interleaved v_max3 chains (the values are integers read as floats: no NaN to canonicalise)
+      float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[0][8], s[0][9], s[0][10]);
+      float mx2 = max3(s[1][0], s[1][1], s[1][2]), mx3 = max3(s[1][8], s[1][9], s[1][10]);
 #pragma unroll
-    for (int i = 3; i < 7; i += 2) {
-      mx0 = max3(mx0, s[0][i], s[0][i + 1]);
-      mx1 = max3(mx1, s[0][i + 8], s[0][i + 9]);
-      mx2 = max3(mx2, s[1][i], s[1][i + 1]);
-      mx3 = max3(mx3, s[1][i + 8], s[1][i + 9]);
-    }
-    mx0 = max3(mx0, s[0][7], s[0][15]);
-    mx2 = max3(mx2, s[1][7], s[1][15]);
-    float smax = max3(mx0, mx1, mx2);
-    smax = max3(smax, mx3, mx3);
-    smax = partner_max(smax);  // still biased by 1.5*2^23
-
-    // Lazy refresh of the running maximum (rare after the first few blocks).  The new maximum
-    // applies to this block's weights at once; O and the row sums, which the pending P.V of the
-    // previous block still has to reach through the stream below, are rescaled after the stream.
-    // Everything that depends on m only (threshold, offsets of the affine maps) is state that changes
-    // on a refresh, so the common path goes from the maximum straight to the comparison.
-    const float m_blk = fmaf(smax, c, nmc);
-    const bool refresh = __ballot(m_blk > m_thr) != 0ull;
+      for (int i = 3; i < 7; i += 2) {
+        mx0 = max3(mx0, s[0][i], s[0][i + 1]);
+        mx1 = max3(mx1, s[0][i + 8], s[0][i + 9]);
+        mx2 = max3(mx2, s[1][i], s[1][i + 1]);
+        mx3 = max3(mx3, s[1][i + 8], s[1][i + 9]);
+      }
+      mx0 = max3(mx0, s[0][7], s[0][15]);
+      mx2 = max3(mx2, s[1][7], s[1][15]);
+      float smax = max3(mx0, mx1, mx2);
+      smax = max3(smax, mx3, mx3);
+      return fmaf(partner_max(smax), c, nmc);
+    };
+    // Refresh of the running maximum: the new maximum applies to this block's weights at once; O and
+    // the row sums, which the pending P.V of the previous block still has to reach through the stream
+    // below, are rescaled after the stream.  Everything that depends on m only (threshold, offsets of
+    // the affine maps) is state that changes here.
     float alpha = 1.0f;
-    if (refresh) {
+    auto apply_refresh = [&](float m_blk) {
       const float m_new = fmaxf(m_i, m_blk);
       alpha = __builtin_amdgcn_exp2f(m_i - m_new);
       m_i = m_new;
       m_thr = m_new + P_HEADROOM;
       m_off = P_EXP_OFFSET - m_new;
-      m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT) * (1.0f / 65535.0f);
+      m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT) * (1.0f / 32767.0f);
       bias = fmaf(-S_MAGIC_F, c, m_off);
       bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
       if constexpr (LSE) d_exact *= alpha;
+    };
+    // Exact path: lazy refresh decided up front from the block maximum (P~ <= 2^(OFFSET + HEADROOM)).
+    // Fast path: optimistic, see below.
+    constexpr bool OPTIMISTIC = !EXACT;
+    bool refresh = false;
+    if constexpr (!OPTIMISTIC) {
+      const float m_blk = block_max();
+      refresh = __ballot(m_blk > m_thr) != 0ull;
+      if (refresh) apply_refresh(m_blk);
     }
 
     // -- the softmax weights of this block in 8 chunks (one 32-bit word of four e4m3 values each);
@@ -487,64 +511,95 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
         read_k_frag(sk1, 2 * r);
         read_k_frag(sk1, 2 * r + 1);
       }
-      if constexpr (D == 64) {
-        if (r == 2) pv_one(pf_p, 2);
-        else if (r == 3) qk_one(0);
-        else if (r == 4) qk_one(1);
-        else if (r == 7) { qk_one(2); qk_one(3); }
-      } else {
-        if (r == 3) pv_one(pf_p, 4);
-        else if (r == 4) { qk_one(0); qk_one(1); }
-        else if (r == 5) qk_one(2);
-        else if (r == 6) qk_one(3);
-        else if (r == 7) { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
+      if (r == DT_TILES - 1 + (D == 64)) pv_one(pf_p, DT_TILES);   // row sums: chunk 2 (D = 64) / 3 (D = 128)
+      if constexpr (!OPTIMISTIC) {
+        if constexpr (D == 64) {
+          if (r == 3) qk_one(0);
+          else if (r == 4) qk_one(1);
+          else if (r == 7) { qk_one(2); qk_one(3); }
+        } else {
+          if (r == 4) { qk_one(0); qk_one(1); }
+          else if (r == 5) qk_one(2);
+          else if (r == 6) qk_one(3);
+          else if (r == 7) { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
+        }
       }
     };
     // Fast path: the e4m3 byte of 2^t is built directly: byte = round(8*(t + 7) + FAST_EXP_SHIFT), i.e.
     // exponent field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of
     // two (at most 6 % off, shifted to be centred).  Per word of four weights: four fmas (the affine
-    // map pre-divided by 65535), two v_cvt_pknorm_u16_f32 (each rounds two values to 16-bit integer
-    // fields, clamping negatives, i.e. masked and underflowing elements, to 0) and one shift-or that
-    // interleaves the two pairs into bytes; the lazy maximum keeps every value <= 126, so no field
-    // spills into its neighbour.  Instead of fma + v_exp_f32 + half a packed FP8 conversion per weight.
-    // Chunk r = word r%4 of row tile r/4.
-    float u_cur[4], u_nxt[4];
-    if constexpr (!EXACT) {
+    // map pre-divided by 32767, result clamped to [0,1], which sends masked and underflowing elements to
+    // 0), two v_cvt_pknorm_i16_f32 (each rounds two values to 16-bit integer fields) and one shift-or
+    // that interleaves the two pairs into bytes.  Instead of fma + v_exp_f32 + half a packed FP8
+    // conversion per weight.  Chunk r = word r%4 of row tile r/4.
+    //
+    // It is optimistic about the maximum: the weights are computed with the running maximum as it
+    // is, and a packed 3-input maximum per chunk keeps the largest field seen.  A field above 126
+    // (the code of 448, the largest e4m3 value; fields cannot exceed 0x7FFF) means some score was more
+    // than 3.8 octaves above the running maximum: only then, and on the first block, is the block
+    // maximum searched (17 v_max3 otherwise spent on every block), the maximum refreshed and the
+    // eight words computed again.  For this the S^T MFMAs of the next block, which overwrite the
+    // scores, are all issued after the check.
+    auto fast_words = [&](auto&& after_chunk, int& ovf) {
+      float u_cur[4], u_nxt[4];
 #pragma unroll
-      for (int q = 0; q < 4; q++) u_cur[q] = fmaf(s[0][q], c8, bias8);
+      for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], c8, bias8);
       __builtin_amdgcn_sched_barrier(0);
-    }
 #pragma unroll
-    for (int r = 0; r < 8; r++) {
-      const int mt = r >> 2, i0 = 4 * (r & 3);
-      int w;
-      if constexpr (!EXACT) {
+      for (int r = 0; r < 8; r++) {
         // the fmas of the next chunk are issued between this chunk's conversions: every conversion
         // finds its input ready
         const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
-        if (rn < 8) { u_nxt[0] = fmaf(s[mtn][in0 + 0], c8, bias8); u_nxt[2] = fmaf(s[mtn][in0 + 2], c8, bias8); }
-        const int lo = cvt_pknorm_u16(u_cur[0], u_cur[2]);
+        if (rn < 8) {
+          u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
+          u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8, bias8);
+        }
+        const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
         __builtin_amdgcn_sched_barrier(0);
-        if (rn < 8) { u_nxt[1] = fmaf(s[mtn][in0 + 1], c8, bias8); u_nxt[3] = fmaf(s[mtn][in0 + 3], c8, bias8); }
-        const int hi = cvt_pknorm_u16(u_cur[1], u_cur[3]);
+        if (rn < 8) {
+          u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
+          u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8, bias8);
+        }
+        const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
         __builtin_amdgcn_sched_barrier(0);
-        w = lshl8_or(hi, lo);
+        pf[r] = lshl8_or(hi, lo);
+        ovf = pk_max3_fields(ovf, lo, hi);
 #pragma unroll
         for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
-      } else {
+        __builtin_amdgcn_sched_barrier(0);
+        after_chunk(r);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    if constexpr (OPTIMISTIC) {
+      int ovf = 0;
+      fast_words(mfma_after_chunk, ovf);
+      const unsigned top = max((unsigned)ovf & 0xffffu, (unsigned)ovf >> 16);
+      refresh = it == 0 || __ballot(top > 126u) != 0ull;
+      if (refresh) {
+        apply_refresh(block_max());
+        int ovf2 = 0;
+        fast_words([](int) {}, ovf2);
+      }
+      qk_mfma();
+    } else {
+#pragma unroll
+      for (int r = 0; r < 8; r++) {
+        const int mt = r >> 2, i0 = 4 * (r & 3);
         // P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential, then the packed FP8 conversion
         const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
         const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
         const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
         const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
         if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
+        int w;
         cvt_pk_fp8<false>(w, p0, p1);
         cvt_pk_fp8<true>(w, p2, p3);
+        pf[r] = w;
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_after_chunk(r);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      pf[r] = w;
-      __builtin_amdgcn_sched_barrier(0);
-      mfma_after_chunk(r);
-      __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (LSE) d_exact += rs;
     if (it + 1 < cnt) dump_s(kb_1);
