@@ -35,9 +35,9 @@ PEAK_HBM_GBS = 8000.0
 HEADLINE_DENSITY = 0.3
 DENSITIES = (0.5, 0.3, 0.2)
 # HBM bytes per attention-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/path_kernels_cogvideox5b_hbm_traffic.txt): FETCH_SIZE 165562 x 2.0 KiB + WRITE_SIZE 213668 x 1.0 KiB,
+# (profiles/path_kernels_cogvideox5b_hbm_traffic.txt): FETCH_SIZE 166963 x 2.0 KiB + WRITE_SIZE 213836 x 1.0 KiB,
 # the factors being what the same counters read for a plain copy of known size; the same at every density
-ATTN_TRAFFIC_BYTES = int((165562 * 2.0 + 213668 * 1.0) * 1024)
+ATTN_TRAFFIC_BYTES = int((166963 * 2.0 + 213836 * 1.0) * 1024)
 
 
 def event_time_ms(fn, reps, warmup):
