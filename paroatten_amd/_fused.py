@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from ._lib import check, load, ptr, stream_of
+from ._lib import ptr, stream_of
 
 _HALF = (torch.float16, torch.bfloat16)
 

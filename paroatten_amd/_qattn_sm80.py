@@ -21,7 +21,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from ._lib import check, load, ptr, stream_of
+from ._lib import load, ptr, stream_of
 
 
 def _chk(cond, msg):

@@ -13,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from ._lib import check, load, ptr, stream_of
+from ._lib import ptr, stream_of
 
 
 def rope_permutation(Q: torch.Tensor, K: torch.Tensor, freq: torch.Tensor, permutation: bool):

@@ -12,7 +12,7 @@ from typing import NamedTuple, Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from ._lib import check, load, ptr, stream_of
+from ._lib import load, ptr, stream_of
 
 # index -> order of the (F,H,W) axes, and the inverse orders (cogvideox.py:38-45, :85-92)
 PERMUTATIONS = ((0, 1, 2), (0, 2, 1), (1, 2, 0), (1, 0, 2), (2, 1, 0), (2, 0, 1))

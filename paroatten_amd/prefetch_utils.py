@@ -18,7 +18,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from ._lib import check, load, ptr
+from ._lib import load, ptr
 
 try:  # diffusers is optional: the callback only needs its calling convention
     from diffusers.callbacks import PipelineCallback as _CallbackBase

@@ -8,7 +8,7 @@ from typing import Optional
 import torch
 
 from . import _fused, _lib
-from ._lib import check, load, ptr, stream_of
+from ._lib import load, ptr, stream_of
 
 
 def _dims(t: torch.Tensor, tensor_layout: str):

@@ -10,9 +10,8 @@ int[L,H], 'empty': bool[L,H]}`, masks bool [H, nb, nb] in the permuted token ord
 """
 from __future__ import annotations
 
-import math
 from dataclasses import dataclass
-from typing import Optional, Tuple
+from typing import Tuple
 
 import torch
 

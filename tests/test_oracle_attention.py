@@ -1,7 +1,6 @@
 """Pins oracle.qk_int32 and oracle.sparse_attention by what they must reduce to: an int64 einsum,
 torch's own softmax/SDPA on dequantised operands, and the invariants of the intended semantics
 (kept blocks form the softmax support; an all-masked row gives 0)."""
-import math
 
 import pytest
 import torch
