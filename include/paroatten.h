@@ -163,7 +163,7 @@ int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, const void* v, 
  *
  * Tokens [0,n_text) are text: copied through.  Image token t = (f*Hh + h)*W + w of head `head`
  * moves to n_text + (c[p0]*S[p1] + c[p1])*S[p2] + c[p2], p = the order `orders[head]` in 0..5
- * (0 FHW, 1 FWH, 2 HWF, 3 HFW, 4 WHF, 5 WFH), S = (F,Hh,W), c = (f,h,w).
+ * (0 FHW, 1 FWH, 2 HWF, 3 HFW, 4 WHF, 5 WFH; any other value is treated as 0), S = (F,Hh,W), c = (f,h,w).
  * paro_rope_permute_fwd: for each of q, k (rotated if cos != NULL) and v (never rotated; any of
  * the three may be NULL): out[b,head,new] = rot(in[b,head,old]).  Rotation of channel pairs:
  *   o[2i] = x[2i]*cos[t,2i] - x[2i+1]*sin[t,2i] ; o[2i+1] = x[2i+1]*cos[t,2i+1] + x[2i]*sin[t,2i+1]

@@ -77,7 +77,8 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
   int n_match = 0;
   for (int bh = 0; bh < BH; bh++) {
     const int b = bh / H, head = bh - b * H;
-    if (orders[head] != order) continue;                  // uniform over the workgroup
+    const int head_order = (unsigned)orders[head] > 5u ? 0 : orders[head];   // as order_strides treats it
+    if (head_order != order) continue;                    // uniform over the workgroup
     if ((n_match++ % head_split) != split) continue;
     float mv[8];
     if (k_mean) {

@@ -10,6 +10,7 @@ constexpr int V_CHUNK = 256;  // tokens per chunk of the per-channel V statistic
 // (0 FHW, 1 FWH, 2 HWF, 3 HFW, 4 WHF, 5 WFH).  Written as selects: a switch that assigns through the
 // three references made the compiler keep them in scratch memory, 12 bytes written per lane and use.
 __device__ __forceinline__ void order_strides(int order, int F, int Hh, int W, int& sf, int& sh, int& sw) {
+  if ((unsigned)order > 5u) order = 0;  // the table lives on the device and cannot be checked by the host
   sf = (order <= 1) ? Hh * W : (order == 3 ? W : (order == 5 ? Hh : 1));
   sh = (order == 2 || order == 3) ? W * F : (order == 0 ? W : (order == 4 ? F : 1));
   sw = (order >= 4) ? Hh * F : (order == 1 ? Hh : (order == 2 ? F : 1));

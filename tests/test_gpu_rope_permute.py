@@ -102,3 +102,21 @@ def test_rope_prototype_module(dev):
             rq, rk = rq.transpose(1, 2), rk.transpose(1, 2)
         assert _ulp_diff(QO.cpu(), rq.reshape(bs, H * W, dim).contiguous()) <= 1
         assert _ulp_diff(KO.cpu(), rk.reshape(bs, H * W, dim).contiguous()) <= 1
+
+
+def test_out_of_range_order_on_device_is_identity(dev):
+    """the order table lives on the device, so the C ABI cannot validate it: a value outside 0..5 is
+    treated as order 0 (no out-of-bounds index can be formed from it) by every kernel that reads it."""
+    from paroatten_amd import permute as PM
+    grid, n_text, D = (2, 3, 4), 8, 64
+    N = n_text + 24
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(1, 2, N, D, generator=g).to(dev, torch.float16)
+    bad = torch.tensor([9, -3], dtype=torch.int32, device=dev)
+    zero = torch.zeros(2, dtype=torch.int32, device=dev)
+    assert torch.equal(PM.permute_index_map(bad, grid), PM.permute_index_map(zero, grid))
+    _, _, v_bad = PM.rope_permute(None, None, x, bad, grid, n_text)
+    assert torch.equal(v_bad, x)
+    assert torch.equal(PM.permute_inverse(x, bad, grid, n_text), x)
+    a, b = PM.rope_permute_quant(x, x, x, bad, grid, n_text), PM.rope_permute_quant(x, x, x, zero, grid, n_text)
+    assert torch.equal(a.q8, b.q8) and torch.equal(a.k_scale, b.k_scale) and torch.equal(a.v8, b.v8)
