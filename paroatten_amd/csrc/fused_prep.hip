@@ -98,9 +98,13 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
       rq[i] = rv;
       rk[i] = rv;
       if (src[i] >= 0) {
-        rq[i] = *reinterpret_cast<const v4i*>(q_in + b * qs_b + head * qs_h + (int64_t)src[i] * qs_n + col);
-        rk[i] = *reinterpret_cast<const v4i*>(k_in + b * ks_b + head * ks_h + (int64_t)src[i] * ks_n + col);
-        rv = *reinterpret_cast<const v4i*>(v_in + b * vs_b + head * vs_h + (int64_t)src[i] * vs_n + col);
+        // read once: non-temporal, the L2 keeps the rotary tables and the V statistics instead
+        rq[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const v4i*>(q_in + b * qs_b + head * qs_h + (int64_t)src[i] * qs_n + col));
+        rk[i] = __builtin_nontemporal_load(
+            reinterpret_cast<const v4i*>(k_in + b * ks_b + head * ks_h + (int64_t)src[i] * ks_n + col));
+        rv = __builtin_nontemporal_load(
+            reinterpret_cast<const v4i*>(v_in + b * vs_b + head * vs_h + (int64_t)src[i] * vs_n + col));
       }
       *reinterpret_cast<v4i*>(&s_tile[(row0 + i * RPI) * PITCH + col]) = rv;
     }
@@ -144,10 +148,12 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(
       }
       if (src[i] >= 0) {
         const int64_t o = ((int64_t)bh * N + kb * 64 + row0 + i * RPI) * D + col;
-        *reinterpret_cast<v2i*>(q8 + o) = v2i{(int)pack4_rint_i8(yq[0], yq[1], yq[2], yq[3]),
-                                              (int)pack4_rint_i8(yq[4], yq[5], yq[6], yq[7])};
-        *reinterpret_cast<v2i*>(k8 + o) = v2i{(int)pack4_rint_i8(yk[0], yk[1], yk[2], yk[3]),
-                                              (int)pack4_rint_i8(yk[4], yk[5], yk[6], yk[7])};
+        __builtin_nontemporal_store(v2i{(int)pack4_rint_i8(yq[0], yq[1], yq[2], yq[3]),
+                                        (int)pack4_rint_i8(yq[4], yq[5], yq[6], yq[7])},
+                                    reinterpret_cast<v2i*>(q8 + o));
+        __builtin_nontemporal_store(v2i{(int)pack4_rint_i8(yk[0], yk[1], yk[2], yk[3]),
+                                        (int)pack4_rint_i8(yk[4], yk[5], yk[6], yk[7])},
+                                    reinterpret_cast<v2i*>(k8 + o));
       }
     }
 
@@ -201,6 +207,8 @@ __global__ void __launch_bounds__(256) rope_k_sum_kernel(const unsigned short* _
       const int bh = bh0 + g;
       if (bh < BH) {
         const int b = bh / H, h = bh - b * H;
+        // ordinary load: K was just written by the projection and is read again by the preparation
+        // pass, so it should stay in the last-level cache
         v4i raw = *reinterpret_cast<const v4i*>(k + b * ks_b + h * ks_h + (int64_t)tok * ks_n + col);
         if (rot) raw = rotate8<DT>(raw, cs, sn);
 #pragma unroll

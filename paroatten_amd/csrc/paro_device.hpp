@@ -120,7 +120,7 @@ __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t*
       p = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], p, true);
       w[g] = p;
     }
-    *reinterpret_cast<v4i*>(ob + (int64_t)c * 16) = v4i{w[0], w[1], w[2], w[3]};
+    __builtin_nontemporal_store(v4i{w[0], w[1], w[2], w[3]}, reinterpret_cast<v4i*>(ob + (int64_t)c * 16));
   }
 }
 

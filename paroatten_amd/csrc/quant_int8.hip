@@ -40,7 +40,8 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(
 #pragma unroll
   for (int i = 0; i < CH; i++) {
     const int tok = g * G + i * ROWS_PER_IT + row0;
-    raw[i] = (tok < N) ? *reinterpret_cast<const v4i*>(xb + (int64_t)tok * xs_n) : v4i{0, 0, 0, 0};
+    raw[i] = (tok < N) ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(xb + (int64_t)tok * xs_n))
+                       : v4i{0, 0, 0, 0};
   }
 
   // value of element (chunk i, slot j) after mean subtraction / scaling; recomputed in the
@@ -74,8 +75,9 @@ __global__ void __launch_bounds__(256) quant_int8_kernel(
 #pragma unroll
     for (int j = 0; j < 8; j++) y[j] = value(i, j) * inv;
     if (tok < N)
-      *reinterpret_cast<v2i*>(ob + (int64_t)tok * os_n) =
-          v2i{(int)pack4_rint_i8(y[0], y[1], y[2], y[3]), (int)pack4_rint_i8(y[4], y[5], y[6], y[7])};
+      __builtin_nontemporal_store(
+          v2i{(int)pack4_rint_i8(y[0], y[1], y[2], y[3]), (int)pack4_rint_i8(y[4], y[5], y[6], y[7])},
+          reinterpret_cast<v2i*>(ob + (int64_t)tok * os_n));
   }
 }
 

@@ -65,17 +65,18 @@ __global__ void __launch_bounds__(256) rope_permute_kernel(
     const int dst = INVERSE ? tok : mapped;
     const int64_t io = b * is_b + head * is_h + (int64_t)src * is_n + col;
     const int64_t oo = b * os_b + head * os_h + (int64_t)dst * os_n + col;
+    // streamed once in, once out: non-temporal on both sides keeps the rotary tables in the L2
     v4i rq, rk, rv;
-    if (q_in) rq = *reinterpret_cast<const v4i*>(q_in + io);
-    if (k_in) rk = *reinterpret_cast<const v4i*>(k_in + io);
-    if (v_in) rv = *reinterpret_cast<const v4i*>(v_in + io);
+    if (q_in) rq = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(q_in + io));
+    if (k_in) rk = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(k_in + io));
+    if (v_in) rv = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(v_in + io));
     if (rope) {
       if (q_in) rq = rotate8<DT>(rq, cs, sn);
       if (k_in) rk = rotate8<DT>(rk, cs, sn);
     }
-    if (q_in) *reinterpret_cast<v4i*>(q_out + oo) = rq;
-    if (k_in) *reinterpret_cast<v4i*>(k_out + oo) = rk;
-    if (v_in) *reinterpret_cast<v4i*>(v_out + oo) = rv;
+    if (q_in) __builtin_nontemporal_store(rq, reinterpret_cast<v4i*>(q_out + oo));
+    if (k_in) __builtin_nontemporal_store(rk, reinterpret_cast<v4i*>(k_out + oo));
+    if (v_in) __builtin_nontemporal_store(rv, reinterpret_cast<v4i*>(v_out + oo));
   }
 }
 
@@ -113,7 +114,8 @@ static int launch_rp(const void* q_in, const void* k_in, const void* v_in, void*
   const int BH = B * H;
   // enough (batch, head) pairs per workgroup to amortise the rotary fragment, few enough that the
   // launch still has several thousand workgroups
-  int hpw = 16;
+  // (without tables there is nothing to amortise: one pair per workgroup, as a plain copy likes it)
+  int hpw = cos_t ? 16 : 1;
   while (hpw > 1 && (int64_t)ceil_div(N, rows) * ceil_div(BH, hpw) < 3072) hpw >>= 1;
   dim3 grid(ceil_div(N, rows), ceil_div(BH, hpw)), block(256);
 #define PARO_RP(DTV, DV)                                                                                          \

@@ -132,7 +132,8 @@ __global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __res
 #pragma unroll
   for (int r = t / LPR; r < 64; r += ROWS) {
     const int tok = kb * 64 + r;
-    const v4i raw = (tok < N) ? *reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n) : v4i{0, 0, 0, 0};
+    const v4i raw = (tok < N) ? __builtin_nontemporal_load(reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n))
+                              : v4i{0, 0, 0, 0};
     *reinterpret_cast<v4i*>(&tile[r * PITCH + col]) = raw;
   }
   __syncthreads();
