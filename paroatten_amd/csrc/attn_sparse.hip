@@ -117,14 +117,6 @@ __device__ __forceinline__ float partner_max(float x) {
   return max3(__uint_as_float(r[0]), __uint_as_float(r[1]), __uint_as_float(r[1]));
 }
 
-__device__ __forceinline__ void* uniform_ptr(const void* ptr) {
-  // the address is the same in every lane; say so, so that the descriptor lives in scalar registers
-  const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
-  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a);
-  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
-  return reinterpret_cast<void*>(((unsigned long long)hi << 32) | lo);
-}
-
 __device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, int voffset, int soffset) {
   // out-of-range bytes read as 0 (raw buffer, bounds-checked by the hardware)
   return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voffset, soffset, 0));
@@ -746,6 +738,17 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
   const int nbq = ceil_div(Nq, 64), nbk = ceil_div(Nk, 64);
   PARO_CHECK(nbk <= 65535, PARO_ERR_RUNTIME, "kv_len %d exceeds 65535 blocks of 64", Nk);
   PARO_CHECK((int64_t)B * H * nbq < (int64_t)1 << 31, PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: too many q-blocks");
+  // one (batch, kv-head) slice of K8 and of V8 is addressed through a buffer descriptor with 32-bit offsets
+  PARO_CHECK(k_stride_n >= D && (int64_t)(Nk - 1) * k_stride_n + D < (int64_t)1 << 31 &&
+                 (int64_t)nbk * 64 * D < (int64_t)1 << 31,
+             PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: one head of key/value spans 2 GiB or more (kv_len %d, stride %lld)",
+             Nk, (long long)k_stride_n);
+  // ring stages + the list of kept blocks (6 bytes each) have to fit the 160 KB of LDS of one CU
+  {
+    const int64_t ring = D == 128 ? 2 * 2 * 64 * 128 : 3 * 2 * 64 * 64;
+    PARO_CHECK(ring + ((int64_t)nbk + 8) * 6 + 64 <= 160 * 1024, PARO_ERR_RUNTIME,
+               "kv_len %d: the list of %d key blocks does not fit the local data share", Nk, nbk);
+  }
   AttnParams p;
   p.q8 = q8; p.k8 = k8; p.v8 = v8; p.q_scale = q_scale; p.k_scale = k_scale; p.v_scale = v_scale; p.v_mean = v_mean;
   p.sparse = sparse; p.out = out; p.lse = lse; p.s_dump = s_dump; p.sparse_bs = sparse_batch_stride;

@@ -22,147 +22,275 @@
 
 namespace paro {
 
+// LDS of the preparation kernel.  The gathered token rows never pass through registers on their way
+// in: LDS-DMA buffer loads drop them into a ring of four 64-token tile slots, Q, K, V of one (batch,
+// head) pair after the other, and the loads of the NEXT pair are issued while this one is rotated,
+// reduced and quantised - three tiles are in flight per workgroup at any time.
+template <int D> struct PrepLds {
+  static constexpr int TILE = 64 * D * 2;          // one tile: 64 rows of D 16-bit values
+  static constexpr int RING = 4;
+  static constexpr int KM_OFF = RING * TILE;       // [2][256 B]  K mean row of this / the next pair
+  static constexpr int ST_OFF = KM_OFF + 2 * 256;  // [2][1 KB]   V reciprocal scale and mean rows
+  static constexpr int LIST_OFF = ST_OFF + 2 * 1024;
+  static constexpr int MAX_PAIRS = 2048;           // (batch, head) pairs one workgroup walks over
+  static constexpr int BYTES = LIST_OFF + MAX_PAIRS * 2;
+  // 16-byte chunk c of tile row `row` sits at chunk position c ^ swz(row): rows r and r + 4, which
+  // the two halves of a wave read together when the V tile is transposed, land on different banks
+  static __device__ __forceinline__ int swz(int row) { return ((row >> 2) & 1) << 2; }
+};
+
+struct PrepParams {
+  const unsigned short *q, *k, *v;
+  const float *cos_t, *sin_t;
+  const int* orders;
+  const unsigned short* k_mean;
+  int8_t* q8;
+  float* q_scale;
+  int8_t* k8;
+  float* k_scale;
+  uint8_t* v8;
+  const float* v_stats;  // per (batch, head): D reciprocal scales, then D means, at v_recp_offset
+  int BH, H, N, nb, n_text, F, Hh, W, head_split;
+  int64_t qs_b, qs_h, qs_n, ks_b, ks_h, ks_n, vs_b, vs_h, vs_n, ms_b, ms_h;
+};
+
+// out-of-range bytes of a raw buffer read as 0 and are not written: `bytes` = 0 switches a whole
+// access off without a branch
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(uniform_ptr(base), 0, bytes, 0x00020000);
+}
+
+// LDS-DMA: 16 (or 4) bytes per lane from a buffer straight into LDS at lds + lane*16 (lane*4); no
+// registers, no ds_write; completion is counted with the wave's other vector-memory operations
+__device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds, int voffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16, voffset, 0, 0, 0);
+}
+__device__ __forceinline__ void buffer_load4_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds, int voffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 4, voffset, 0, 0, 0);
+}
+
+// waits until at most N of this wave's vector-memory operations are outstanding (they complete in
+// issue order) and all of its LDS operations are done
+template <int N> __device__ __forceinline__ void wait_vm() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(N) : "memory");
+}
+
 template <int DT, int D>
-__global__ void __launch_bounds__(256) rope_permute_quant_kernel(
-    const unsigned short* __restrict__ q_in, const unsigned short* __restrict__ k_in,
-    const unsigned short* __restrict__ v_in, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-    const int* __restrict__ orders, const unsigned short* __restrict__ k_mean, int8_t* __restrict__ q8,
-    float* __restrict__ q_scale, int8_t* __restrict__ k8, float* __restrict__ k_scale, uint8_t* __restrict__ v8,
-    const float* __restrict__ v_recp, const float* __restrict__ v_mean, int BH, int H, int N, int nb, int n_text,
-    int F, int Hh, int W, int head_split, int64_t qs_b, int64_t qs_h, int64_t qs_n, int64_t ks_b, int64_t ks_h,
-    int64_t ks_n, int64_t vs_b, int64_t vs_h, int64_t vs_n, int64_t ms_b, int64_t ms_h) {
+__global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParams p) {
+  using L = PrepLds<D>;
   constexpr int LPR = D / 8;            // lanes per token row (16-byte pieces)
   constexpr int RPI = 64 / LPR;         // rows one wave covers per load instruction
-  constexpr int PC = 16 / RPI;          // pieces per lane: a wave owns 16 rows of the block
-  constexpr int PITCH = D + 8;          // V tile row pitch in 16-bit elements
+  constexpr int PC = 16 / RPI;          // pieces per lane and tile: a wave owns 16 rows of the block
+  constexpr int NV = D == 128 ? 2 : 1;  // distinct channel offsets among a lane's pieces
+  // vector-memory operations one wave issues per pair: PC per tile, two more with the K tile (mean
+  // row, V statistics row), and ST stores that are issued unconditionally (q8, k8: PC each, v8: D/64)
+  constexpr int ST = 2 * PC + D / 64;
+  constexpr int OOB = 0x7ffffff0;       // offset beyond any descriptor range
+
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  unsigned short* s_list = reinterpret_cast<unsigned short*>(smem + L::LIST_OFF);
   __shared__ int s_src[64];             // source token of each destination row, -1 past the end
-  __shared__ __attribute__((aligned(16))) unsigned short s_tile[64 * PITCH];
   __shared__ float s_amax[2][4];        // [q|k][wave]
+  __shared__ int s_npairs;
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int kb = blockIdx.x;
   const int order = blockIdx.y % 6, split = blockIdx.y / 6;
-  const bool rope = cos_t != nullptr;
+  const bool rope = p.cos_t != nullptr;
 
   if (t < 64) {
     const int d = kb * 64 + t;
     int src = -1;
-    if (d < N) src = d < n_text ? d : n_text + unpermute_index(d - n_text, order, F, Hh, W);
+    if (d < p.N) src = d < p.n_text ? d : p.n_text + unpermute_index(d - p.n_text, order, p.F, p.Hh, p.W);
     s_src[t] = src;
   }
+  if (wave == 1) {
+    // the (batch, head) pairs whose head uses this workgroup's order, every head_split-th of them
+    int cnt = 0;
+    for (int base = 0; base < p.BH; base += 64) {
+      const int bh = base + lane;
+      bool match = false;
+      if (bh < p.BH) {
+        const int o = p.orders[bh % p.H];
+        match = ((unsigned)o > 5u ? 0 : o) == order;   // as order_strides treats it
+      }
+      const unsigned long long bal = __ballot(match);
+      const int idx = cnt + __popcll(bal & ((1ull << lane) - 1ull));
+      if (match && idx % p.head_split == split) s_list[idx / p.head_split] = (unsigned short)bh;
+      cnt += __popcll(bal);
+    }
+    if (lane == 0) s_npairs = cnt > split ? (cnt - split + p.head_split - 1) / p.head_split : 0;
+  }
   __syncthreads();
+  const int npairs = s_npairs;
+  if (npairs == 0) return;
 
-  // this lane's pieces: rows 16*wave + i*RPI + lane/LPR of the block, channels col..col+7; their
-  // rotary-table entries stay in registers for every (batch, head) the workgroup walks over
-  const int col = (lane % LPR) * 8;
-  const int row0 = 16 * wave + lane / LPR;
-  int src[PC];
+  // this lane's pieces: tile rows 16*wave + i*RPI + lane/LPR; LDS chunk position lane%LPR of such a
+  // row holds channels col..col+7.  Their rotary-table entries stay in registers for every pair.
+  int src[PC], col[NV], voq[PC], vok[PC], vov[PC];
   float cs[PC][8], sn[PC][8];
 #pragma unroll
   for (int i = 0; i < PC; i++) {
-    src[i] = s_src[row0 + i * RPI];
-    if (rope && src[i] >= n_text) {
-      const int64_t o = (int64_t)(src[i] - n_text) * D + col;
-      const v4f c0 = *reinterpret_cast<const v4f*>(cos_t + o), c1 = *reinterpret_cast<const v4f*>(cos_t + o + 4);
-      const v4f s0 = *reinterpret_cast<const v4f*>(sin_t + o), s1 = *reinterpret_cast<const v4f*>(sin_t + o + 4);
+    const int row = 16 * wave + i * RPI + lane / LPR;
+    const int c = ((lane % LPR) ^ L::swz(row)) * 8;
+    if (i < NV) col[i] = c;
+    src[i] = s_src[row];
+    voq[i] = vok[i] = vov[i] = OOB;
+    if (src[i] >= 0) {
+      voq[i] = (int)(((int64_t)src[i] * p.qs_n + c) * 2);
+      vok[i] = (int)(((int64_t)src[i] * p.ks_n + c) * 2);
+      vov[i] = (int)(((int64_t)src[i] * p.vs_n + c) * 2);
+    }
+  }
+  const int n_chunks = (p.N + V_CHUNK - 1) / V_CHUNK;
+  const int q_bytes = (int)((((int64_t)p.N - 1) * p.qs_n + D) * 2);
+  const int k_bytes = (int)((((int64_t)p.N - 1) * p.ks_n + D) * 2);
+  const int v_bytes = (int)((((int64_t)p.N - 1) * p.vs_n + D) * 2);
+
+  // ---- tile movers: every wave fetches the 16 rows it will itself rotate and quantise, so Q and K
+  //      need no barrier, only the wave's own wait; the V tile is read across waves -----------------
+  auto load_tile = [&](const unsigned short* base, int bytes, const int* voff, int slot) {
+    const __amdgpu_buffer_rsrc_t r = raw_buffer(base, bytes);
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        cs[i][j] = c0[j]; cs[i][4 + j] = c1[j];
-        sn[i][j] = s0[j]; sn[i][4 + j] = s1[j];
+    for (int i = 0; i < PC; i++)
+      buffer_load16_lds(r, smem + slot * L::TILE + (wave_u * PC + i) * 1024, voff[i]);
+  };
+  // the pair the loads are issued for: (batch nx_b, head nx_h), or none (nx_bh < 0): the loads are
+  // still issued then (the wait counts stay the same) but fetch nothing
+  int nx_bh, nx_b = 0, nx_h = 0;
+  auto set_next = [&](int bh) {
+    nx_bh = bh;
+    if (bh >= 0) { nx_b = bh / p.H; nx_h = bh - nx_b * p.H; }
+  };
+  auto load_q = [&](int slot) {
+    load_tile(p.q + nx_b * p.qs_b + nx_h * p.qs_h, nx_bh < 0 ? 0 : q_bytes, voq, slot);
+  };
+  auto load_k = [&](int slot, int par) {
+    const int bh = nx_bh, b = nx_b, head = nx_h;
+    load_tile(p.k + b * p.ks_b + head * p.ks_h, bh < 0 ? 0 : k_bytes, vok, slot);
+    // the pair's K mean row (zeros without smoothing) and its V statistics: every wave fetches the
+    // same bytes to the same place
+    const bool km = bh >= 0 && p.k_mean != nullptr;
+    const __amdgpu_buffer_rsrc_t rm = raw_buffer(km ? p.k_mean + b * p.ms_b + head * p.ms_h : p.k, km ? D * 2 : 0);
+    buffer_load4_lds(rm, smem + L::KM_OFF + par * 256, lane * 4);
+    const __amdgpu_buffer_rsrc_t rs =
+        raw_buffer(bh < 0 ? p.v_stats : p.v_stats + v_recp_offset(bh, n_chunks, D), bh < 0 ? 0 : 2 * D * 4);
+    buffer_load16_lds(rs, smem + L::ST_OFF + par * 1024, lane * 16);
+  };
+  auto load_v = [&](int slot) {
+    load_tile(p.v + nx_b * p.vs_b + nx_h * p.vs_h, nx_bh < 0 ? 0 : v_bytes, vov, slot);
+  };
+  auto own_piece = [&](int slot, int i) {
+    return *reinterpret_cast<const v4i*>(smem + slot * L::TILE + (wave_u * PC + i) * 1024 + lane * 16);
+  };
+
+  set_next(__builtin_amdgcn_readfirstlane((int)s_list[0]));
+  load_q(0);
+  load_k(1, 0);
+  load_v(2);
+  // the table entries are fetched behind the first pair's tiles and pinned down here, so that nothing
+  // but the tile stream is outstanding once the loop runs
+#pragma unroll
+  for (int i = 0; i < PC; i++) {
+    if (rope && src[i] >= p.n_text) {
+      const int64_t o = (int64_t)(src[i] - p.n_text) * D + col[i % NV];
+      const v4f c0 = *reinterpret_cast<const v4f*>(p.cos_t + o), c1 = *reinterpret_cast<const v4f*>(p.cos_t + o + 4);
+      const v4f s0 = *reinterpret_cast<const v4f*>(p.sin_t + o), s1 = *reinterpret_cast<const v4f*>(p.sin_t + o + 4);
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        cs[i][e] = c0[e]; cs[i][4 + e] = c1[e];
+        sn[i][e] = s0[e]; sn[i][4 + e] = s1[e];
       }
     }
   }
-
-  const int n_chunks = (N + V_CHUNK - 1) / V_CHUNK;
-  int n_match = 0;
-  for (int bh = 0; bh < BH; bh++) {
-    const int b = bh / H, head = bh - b * H;
-    const int head_order = (unsigned)orders[head] > 5u ? 0 : orders[head];   // as order_strides treats it
-    if (head_order != order) continue;                    // uniform over the workgroup
-    if ((n_match++ % head_split) != split) continue;
-    float mv[8];
-    if (k_mean) {
-      const v4i m = *reinterpret_cast<const v4i*>(k_mean + b * ms_b + head * ms_h + col);
 #pragma unroll
-      for (int j = 0; j < 8; j++) mv[j] = elem16_to_f32<DT>(m, j);
-    } else {
+  for (int i = 0; i < PC; i++)
 #pragma unroll
-      for (int j = 0; j < 8; j++) mv[j] = 0.f;
-    }
+    for (int e = 0; e < 8; e++) asm volatile("" : "+v"(cs[i][e]), "+v"(sn[i][e]));
+  int j = 0;  // ring position of the current pair's Q tile (tile number mod 4)
+  for (int ip = 0; ip < npairs; ip++) {
+    const int bh = nx_bh;
+    set_next(ip + 1 < npairs ? __builtin_amdgcn_readfirstlane((int)s_list[ip + 1]) : -1);
+    const int par = ip & 1;
 
-    // ---- gather; rotate Q and K and round them to the input type (kept packed); V to the tile ----
+    // ---- Q tile: wait for this wave's rows; the barrier says every wave has finished with the V
+    //      tile of the previous pair, whose slot the next Q tile is fetched into -------------------
+    if (ip == 0) wait_vm<2 * PC + 2>(); else wait_vm<2 * PC + 2 + ST>();
+    __builtin_amdgcn_s_barrier();
+    load_q((j + 3) & 3);
     v4i rq[PC], rk[PC];
-#pragma unroll
-    for (int i = 0; i < PC; i++) {
-      v4i rv = {0, 0, 0, 0};
-      rq[i] = rv;
-      rk[i] = rv;
-      if (src[i] >= 0) {
-        // read once: non-temporal, the L2 keeps the rotary tables and the V statistics instead
-        rq[i] = __builtin_nontemporal_load(
-            reinterpret_cast<const v4i*>(q_in + b * qs_b + head * qs_h + (int64_t)src[i] * qs_n + col));
-        rk[i] = __builtin_nontemporal_load(
-            reinterpret_cast<const v4i*>(k_in + b * ks_b + head * ks_h + (int64_t)src[i] * ks_n + col));
-        rv = __builtin_nontemporal_load(
-            reinterpret_cast<const v4i*>(v_in + b * vs_b + head * vs_h + (int64_t)src[i] * vs_n + col));
-      }
-      *reinterpret_cast<v4i*>(&s_tile[(row0 + i * RPI) * PITCH + col]) = rv;
-    }
     float aq = 0.0000001f, ak = 0.0000001f;
 #pragma unroll
     for (int i = 0; i < PC; i++) {
-      if (rope && src[i] >= n_text) {
-        rq[i] = rotate8<DT>(rq[i], cs[i], sn[i]);
-        rk[i] = rotate8<DT>(rk[i], cs[i], sn[i]);
-      }
-      if (src[i] >= 0) {  // rows past the end count as zero, whatever the mean
+      rq[i] = own_piece(j & 3, i);
+      if (rope && src[i] >= p.n_text) rq[i] = rotate8<DT>(rq[i], cs[i], sn[i]);
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-          aq = fmaxf(aq, fabsf(elem16_to_f32<DT>(rq[i], j)));
-          ak = fmaxf(ak, fabsf(elem16_to_f32<DT>(rk[i], j) - mv[j]));
-        }
-      }
+      for (int e = 0; e < 8; e++) aq = fmaxf(aq, fabsf(elem16_to_f32<DT>(rq[i], e)));   // rows past the end are 0
     }
     aq = wave_max(aq);
-    ak = wave_max(ak);
-    if (lane == 0) {
-      s_amax[0][wave] = aq;
-      s_amax[1][wave] = ak;
-    }
-    __syncthreads();
+    if (lane == 0) s_amax[0][wave] = aq;
 
-    // ---- group maxima: Q per 32 rows (two waves), K per 64 rows (the workgroup) --------------
-    aq = fmaxf(s_amax[0][wave & 2], s_amax[0][(wave & 2) + 1]);
-    ak = fmaxf(fmaxf(s_amax[1][0], s_amax[1][1]), fmaxf(s_amax[1][2], s_amax[1][3]));
-    if (lane == 0 && (wave & 1) == 0) q_scale[(int64_t)bh * (nb * 2) + kb * 2 + (wave >> 1)] = aq / 127.0f;
-    if (t == 0) k_scale[(int64_t)bh * nb + kb] = ak / 127.0f;
-    const float inv_q = 127.0f / aq, inv_k = 127.0f / ak;
+    // ---- K tile (its slot's next tenant is fetched by the same wave into the same rows) ---------
+    if (ip == 0) wait_vm<2 * PC>(); else wait_vm<2 * PC + ST>();
+    load_k(j & 3, par ^ 1);
+    float mv[NV][8];
+#pragma unroll
+    for (int n = 0; n < NV; n++) {
+      const v4i m = *reinterpret_cast<const v4i*>(smem + L::KM_OFF + par * 256 + col[n] * 2);
+#pragma unroll
+      for (int e = 0; e < 8; e++) mv[n][e] = elem16_to_f32<DT>(m, e);
+    }
 #pragma unroll
     for (int i = 0; i < PC; i++) {
-      // |x * (127/amax)| <= 127 up to rounding: the reference's clamp to [-128,127] never acts
-      float yq[8], yk[8];
+      rk[i] = own_piece((j + 1) & 3, i);
+      if (rope && src[i] >= p.n_text) rk[i] = rotate8<DT>(rk[i], cs[i], sn[i]);
+      if (src[i] >= 0) {  // rows past the end count as zero, whatever the mean
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        yq[j] = elem16_to_f32<DT>(rq[i], j) * inv_q;
-        yk[j] = (elem16_to_f32<DT>(rk[i], j) - mv[j]) * inv_k;
-      }
-      if (src[i] >= 0) {
-        const int64_t o = ((int64_t)bh * N + kb * 64 + row0 + i * RPI) * D + col;
-        __builtin_nontemporal_store(v2i{(int)pack4_rint_i8(yq[0], yq[1], yq[2], yq[3]),
-                                        (int)pack4_rint_i8(yq[4], yq[5], yq[6], yq[7])},
-                                    reinterpret_cast<v2i*>(q8 + o));
-        __builtin_nontemporal_store(v2i{(int)pack4_rint_i8(yk[0], yk[1], yk[2], yk[3]),
-                                        (int)pack4_rint_i8(yk[4], yk[5], yk[6], yk[7])},
-                                    reinterpret_cast<v2i*>(k8 + o));
+        for (int e = 0; e < 8; e++) ak = fmaxf(ak, fabsf(elem16_to_f32<DT>(rk[i], e) - mv[i % NV][e]));
       }
     }
+    ak = wave_max(ak);
+    if (lane == 0) s_amax[1][wave] = ak;
 
-    // ---- V tile -> e4m3 fragments -------------------------------------------------------------
-    pack_v_tile<DT, D, PITCH>(s_tile, v8 + ((int64_t)bh * nb + kb) * (int64_t)(64 * D),
-                              v_recp + v_recp_offset(bh, n_chunks, D), v_mean ? v_mean + (int64_t)bh * D : nullptr,
-                              kb * 64, N, t);
-    __syncthreads();  // the tile and s_amax are reused by the next (batch, head)
+    // ---- V tile: landed in every wave, and the group maxima are visible ------------------------
+    if (ip == 0) wait_vm<2 * PC + 2>(); else wait_vm<2 * PC + 2 + ST>();
+    __builtin_amdgcn_s_barrier();
+    load_v((j + 1) & 3);
+    // group maxima: Q per 32 rows (two waves), K per 64 rows (the workgroup)
+    aq = fmaxf(s_amax[0][wave & 2], s_amax[0][(wave & 2) + 1]);
+    ak = fmaxf(fmaxf(s_amax[1][0], s_amax[1][1]), fmaxf(s_amax[1][2], s_amax[1][3]));
+    if (lane == 0 && (wave & 1) == 0) p.q_scale[(int64_t)bh * (p.nb * 2) + kb * 2 + (wave >> 1)] = aq / 127.0f;
+    if (t == 0) p.k_scale[(int64_t)bh * p.nb + kb] = ak / 127.0f;
+    const float inv_q = 127.0f / aq, inv_k = 127.0f / ak;
+    {
+      // rows >= N fall outside the descriptor and are not written
+      const __amdgpu_buffer_rsrc_t rq8 = raw_buffer(p.q8 + (int64_t)bh * p.N * D, p.N * D);
+      const __amdgpu_buffer_rsrc_t rk8 = raw_buffer(p.k8 + (int64_t)bh * p.N * D, p.N * D);
+#pragma unroll
+      for (int i = 0; i < PC; i++) {
+        // |x * (127/amax)| <= 127 up to rounding: the reference's clamp to [-128,127] never acts
+        float yq[8], yk[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          yq[e] = elem16_to_f32<DT>(rq[i], e) * inv_q;
+          yk[e] = (elem16_to_f32<DT>(rk[i], e) - mv[i % NV][e]) * inv_k;
+        }
+        const int o = (kb * 64 + 16 * wave + i * RPI + lane / LPR) * D + col[i % NV];
+        __builtin_amdgcn_raw_buffer_store_b64(
+            v2u{pack4_rint_i8(yq[0], yq[1], yq[2], yq[3]), pack4_rint_i8(yq[4], yq[5], yq[6], yq[7])}, rq8, o, 0, 2);
+        __builtin_amdgcn_raw_buffer_store_b64(
+            v2u{pack4_rint_i8(yk[0], yk[1], yk[2], yk[3]), pack4_rint_i8(yk[4], yk[5], yk[6], yk[7])}, rk8, o, 0, 2);
+      }
+    }
+    // V tile -> e4m3 fragments
+    const float* st = reinterpret_cast<const float*>(smem + L::ST_OFF + par * 1024);
+    pack_v_tile<DT, D, D, true>(reinterpret_cast<const unsigned short*>(smem + ((j + 2) & 3) * L::TILE),
+                                p.v8 + ((int64_t)bh * p.nb + kb) * (int64_t)(64 * D), st, st + D, kb * 64, p.N, t);
+    j = (j + 3) & 3;
   }
+  // the loads issued for the pair after the last one fetch nothing, but they do write LDS
+  wait_vm<0>();
 }
 
 // K mean over tokens AFTER the rotation (the permutation does not change a mean): partial sums per
@@ -257,9 +385,21 @@ __global__ void __launch_bounds__(1024) k_mean_finalize_kernel(const float* __re
   }
 }
 
+template <int DT, int D>
+static int launch_prep(const PrepParams& p, dim3 grid, hipStream_t st) {
+  auto kern = rope_permute_quant_kernel<DT, D>;
+  constexpr int lds = PrepLds<D>::BYTES;
+  if (lds > 48 * 1024)
+    PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, p);
+  return PARO_OK;
+}
+
 static int check_prep(const char* fn, int dtype, int B, int H, int N, int D, int n_text, int F, int Hh, int W,
                       int64_t s_b, int64_t s_h, int64_t s_n) {
   PARO_CHECK(B > 0 && H > 0 && N > 0, PARO_ERR_RUNTIME, "%s: empty shape", fn);
+  PARO_CHECK((int64_t)B * H <= MAX_GRID_YZ, PARO_ERR_RUNTIME, "%s: batch * heads = %lld exceeds %d", fn,
+             (long long)B * H, MAX_GRID_YZ);
   PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
   PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
              "Unsupported input dtype (expect float16 or bfloat16)");
@@ -344,6 +484,12 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
   PARO_CHECK(workspace_bytes >= paro_prep_workspace_bytes(B, H, N, D) && ((uintptr_t)workspace % 16) == 0,
              PARO_ERR_RUNTIME, "paro_rope_permute_quant_fwd: workspace of %lld bytes is too small or misaligned",
              (long long)workspace_bytes);
+  // one (batch, head) slice of each input and of q8 / k8 is addressed through 32-bit buffer offsets
+  PARO_CHECK(q_stride_n >= D && k_stride_n >= D && v_stride_n >= D &&
+                 ((int64_t)N - 1) * q_stride_n + D < (int64_t)1 << 30 &&
+                 ((int64_t)N - 1) * k_stride_n + D < (int64_t)1 << 30 &&
+                 ((int64_t)N - 1) * v_stride_n + D < (int64_t)1 << 30,
+             PARO_ERR_RUNTIME, "paro_rope_permute_quant_fwd: one head of q, k or v spans 2 GiB or more");
   hipStream_t st = (hipStream_t)stream;
   // V statistics do not depend on the token order: taken on the unpermuted tensor
   if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, (float*)workspace, B, H, N, D, v_stride_b, v_stride_h,
@@ -355,20 +501,26 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
   // workgroup holds are reused
   int head_split = 1;
   while (head_split < 8 && (int64_t)nb * 6 * head_split < 2048 && head_split * 2 <= B * H) head_split *= 2;
-  dim3 grid(nb, 6 * head_split), block(256);
-#define PARO_PREP(DTV, DV)                                                                                      \
-  hipLaunchKernelGGL((rope_permute_quant_kernel<DTV, DV>), grid, block, 0, st, (const unsigned short*)q,        \
-                     (const unsigned short*)k, (const unsigned short*)v, cos, sin, (const int*)orders,          \
-                     (const unsigned short*)k_mean, q8, q_scale, k8, k_scale, v8, (const float*)workspace,      \
-                     (const float*)(smooth_v ? v_mean : nullptr), B * H, H, N, nb, n_text, F, Hh, W, head_split, \
-                     q_stride_b, q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n, v_stride_b,        \
-                     v_stride_h, v_stride_n, mean_stride_b, mean_stride_h)
+  while (ceil_div(B * H, head_split) > PrepLds<64>::MAX_PAIRS) head_split *= 2;   // the list a workgroup keeps in LDS
+  PrepParams p;
+  p.q = (const unsigned short*)q; p.k = (const unsigned short*)k; p.v = (const unsigned short*)v;
+  p.cos_t = cos; p.sin_t = sin; p.orders = (const int*)orders; p.k_mean = (const unsigned short*)k_mean;
+  p.q8 = q8; p.q_scale = q_scale; p.k8 = k8; p.k_scale = k_scale; p.v8 = v8; p.v_stats = (const float*)workspace;
+  p.BH = B * H; p.H = H; p.N = N; p.nb = nb; p.n_text = n_text; p.F = F; p.Hh = Hh; p.W = W; p.head_split = head_split;
+  p.qs_b = q_stride_b; p.qs_h = q_stride_h; p.qs_n = q_stride_n;
+  p.ks_b = k_stride_b; p.ks_h = k_stride_h; p.ks_n = k_stride_n;
+  p.vs_b = v_stride_b; p.vs_h = v_stride_h; p.vs_n = v_stride_n;
+  p.ms_b = mean_stride_b; p.ms_h = mean_stride_h;
+  dim3 grid(nb, 6 * head_split);
+#define PARO_PREP(DTV, DV) rc = launch_prep<DTV, DV>(p, grid, st)
+  int rc;
   if (dtype == PARO_DTYPE_F16) {
     if (D == 64) PARO_PREP(PARO_DTYPE_F16, 64); else PARO_PREP(PARO_DTYPE_F16, 128);
   } else {
     if (D == 64) PARO_PREP(PARO_DTYPE_BF16, 64); else PARO_PREP(PARO_DTYPE_BF16, 128);
   }
 #undef PARO_PREP
+  if (rc) return rc;
   PARO_HIP(hipGetLastError());
   return PARO_OK;
 }

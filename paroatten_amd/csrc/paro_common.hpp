@@ -12,6 +12,7 @@ namespace paro {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -70,5 +71,8 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// batch and head counts become the y / z dimensions of a launch grid (at most 65535 each)
+constexpr int MAX_GRID_YZ = 65535;
 
 }  // namespace paro

@@ -80,6 +80,14 @@ __device__ __forceinline__ v4i rotate8(const v4i raw, const float* cs, const flo
   return o;
 }
 
+__device__ __forceinline__ void* uniform_ptr(const void* ptr) {
+  // the address is the same in every lane; say so, so that the descriptor lives in scalar registers
+  const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a);
+  const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+  return reinterpret_cast<void*>(((unsigned long long)hi << 32) | lo);
+}
+
 // four values y (|y| <= 127.5, not yet rounded) -> four int8 = rint(y) packed in a word.  Adding
 // 1.5*2^23 rounds to the nearest integer, ties to even, exactly as rintf does (the sum lies in
 // [2^23, 2^24), where floats are the integers), and leaves the two's-complement byte in bits 0..7.
@@ -96,12 +104,14 @@ __device__ __forceinline__ unsigned pack4_rint_i8(float y0, float y1, float y2, 
 // e4m3 in the fragment order of the P.V MFMA: 16-byte piece c = (dt, mt, lane) holds channel
 // 32*dt + lane%32 of tokens 32*mt + 8*g + 4*(lane/32) + q, byte 4*g + q.  recp = 448 / max|v - mean|
 // (0 for a constant channel), as MeanScaleKernel of the reference forms it
-// (csrc/fused/fused.cu:399,414).  256 threads.
-template <int DT, int D, int PITCH>
+// (csrc/fused/fused.cu:399,414).  256 threads.  SWZ: rows are unpadded (PITCH = D) and 16-byte chunk c
+// of row r sits at chunk position c ^ 4*((r >> 2) & 1).
+template <int DT, int D, int PITCH, bool SWZ = false>
 __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t* ob, const float* v_recp,
                                             const float* v_mean, int tok0, int N, int t) {
 #pragma unroll
-  for (int c = t; c < 4 * D; c += 256) {
+  for (int n = 0; n < D / 64; n++) {   // 4*D pieces, 256 threads
+    const int c = t + 256 * n;
     const int lane = c & 63, mt = (c >> 6) & 1, dt = c >> 7;
     const int ch = 32 * dt + (lane & 31);
     const float mean = v_mean ? v_mean[ch] : 0.f;
@@ -113,7 +123,8 @@ __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t*
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         const int r = 32 * mt + 8 * g + 4 * (lane >> 5) + q;
-        const float x = F16x<DT>::to_f32(tile[r * PITCH + ch]);
+        const int at = SWZ ? r * PITCH + ((((ch >> 3) ^ (((r >> 2) & 1) << 2)) << 3) | (ch & 7)) : r * PITCH + ch;
+        const float x = F16x<DT>::to_f32(tile[at]);
         f[q] = (tok0 + r < N) ? (x - mean) * rc : 0.f;
       }
       int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);

@@ -132,6 +132,8 @@ extern "C" int paro_quant_int8(const void* x, int dtype, const void* mean, int8_
   using namespace paro;
   PARO_CHECK(x && out && scale, PARO_ERR_RUNTIME, "paro_quant_int8: null tensor pointer");
   PARO_CHECK(B > 0 && H > 0 && N > 0 && n_groups > 0, PARO_ERR_RUNTIME, "paro_quant_int8: empty shape");
+  PARO_CHECK(B <= MAX_GRID_YZ && H <= MAX_GRID_YZ, PARO_ERR_RUNTIME, "paro_quant_int8: batch or head count exceeds %d",
+             MAX_GRID_YZ);
   PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
   PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
              "Unsupported input dtype (expect float16 or bfloat16)");

@@ -94,6 +94,8 @@ __global__ void permute_index_kernel(int* __restrict__ idx, const int* __restric
 static int check_common(const char* fn, int dtype, int B, int H, int N, int D, int n_text, int F, int Hh, int W,
                         int64_t is_b, int64_t is_h, int64_t is_n, int64_t os_b, int64_t os_h, int64_t os_n) {
   PARO_CHECK(B > 0 && H > 0 && N > 0, PARO_ERR_RUNTIME, "%s: empty shape", fn);
+  PARO_CHECK((int64_t)B * H <= MAX_GRID_YZ, PARO_ERR_RUNTIME, "%s: batch * heads = %lld exceeds %d", fn,
+             (long long)B * H, MAX_GRID_YZ);
   PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
   PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
              "Unsupported input dtype (expect float16 or bfloat16)");
@@ -182,6 +184,8 @@ extern "C" int paro_permute_index_map(int32_t* idx, const int32_t* orders, int H
   using namespace paro;
   PARO_CHECK(idx && orders, PARO_ERR_RUNTIME, "paro_permute_index_map: null pointer");
   PARO_CHECK(H > 0 && F > 0 && Hh > 0 && W > 0, PARO_ERR_RUNTIME, "paro_permute_index_map: empty shape");
+  PARO_CHECK(H <= MAX_GRID_YZ && (int64_t)F * Hh * W < (int64_t)1 << 31, PARO_ERR_RUNTIME,
+             "paro_permute_index_map: head count or grid too large");
   const int n = F * Hh * W;
   hipLaunchKernelGGL(permute_index_kernel, dim3(ceil_div(n, 256), H), dim3(256), 0, (hipStream_t)stream, idx,
                      (const int*)orders, F, Hh, W);

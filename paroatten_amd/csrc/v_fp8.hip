@@ -109,8 +109,9 @@ __global__ void __launch_bounds__(1024) v_finalize_kernel(float* partial, float*
     v_scale[bh * D + ch] = amax / 448.0f;
     if (v_mean) v_mean[bh * D + ch] = mean;
     // every thread of this workgroup has read its partials before the barrier above: the head of the
-    // region is free to carry the reciprocal to the pack kernel
+    // region is free to carry the reciprocal, and behind it the mean, to the pack kernel
     partial[v_recp_offset(bh, n_chunks, D) + ch] = amax > 0.f ? 448.0f / amax : 0.f;
+    partial[v_recp_offset(bh, n_chunks, D) + D + ch] = mean;
   }
 }
 
@@ -222,6 +223,8 @@ extern "C" int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_s
   PARO_CHECK(v && v8 && v_scale && partial, PARO_ERR_RUNTIME, "paro_v_fp8_pack: null tensor pointer");
   PARO_CHECK(!smooth || v_mean, PARO_ERR_RUNTIME, "paro_v_fp8_pack: smoothing needs a v_mean buffer");
   PARO_CHECK(B > 0 && Hkv > 0 && N > 0, PARO_ERR_RUNTIME, "paro_v_fp8_pack: empty shape");
+  PARO_CHECK(B <= MAX_GRID_YZ && Hkv <= MAX_GRID_YZ, PARO_ERR_RUNTIME, "paro_v_fp8_pack: batch or head count exceeds %d",
+             MAX_GRID_YZ);
   PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
   PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
              "Unsupported input dtype (expect float16 or bfloat16)");
@@ -247,6 +250,8 @@ extern "C" int paro_sub_mean(const void* v, int dtype, const void* mean, void* o
                              int64_t out_stride_h, int64_t out_stride_n, void* stream) {
   using namespace paro;
   PARO_CHECK(v && mean && out_f16, PARO_ERR_RUNTIME, "paro_sub_mean: null tensor pointer");
+  PARO_CHECK(B > 0 && H > 0 && N > 0 && B <= MAX_GRID_YZ && H <= MAX_GRID_YZ, PARO_ERR_RUNTIME,
+             "paro_sub_mean: empty shape, or batch or head count above %d", MAX_GRID_YZ);
   PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
   PARO_CHECK(dtype == PARO_DTYPE_F16 || dtype == PARO_DTYPE_BF16, PARO_ERR_RUNTIME,
              "Unsupported input dtype (expect float16 or bfloat16)");
