@@ -61,7 +61,11 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t raw_buffer(const void* base, i
 }
 
 // LDS-DMA: 16 (or 4) bytes per lane from a buffer straight into LDS at lds + lane*16 (lane*4); no
-// registers, no ds_write; completion is counted with the wave's other vector-memory operations
+// registers, no ds_write; completion is counted with the wave's other vector-memory operations.  The
+// token rows are read once: non-temporal.
+__device__ __forceinline__ void buffer_load16_lds_once(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds, int voffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16, voffset, 0, 0, 2);
+}
 __device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds, int voffset) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16, voffset, 0, 0, 0);
 }
@@ -154,7 +158,7 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
     const __amdgpu_buffer_rsrc_t r = raw_buffer(base, bytes);
 #pragma unroll
     for (int i = 0; i < PC; i++)
-      buffer_load16_lds(r, smem + slot * L::TILE + (wave_u * PC + i) * 1024, voff[i]);
+      buffer_load16_lds_once(r, smem + slot * L::TILE + (wave_u * PC + i) * 1024, voff[i]);
   };
   // the pair the loads are issued for: (batch nx_b, head nx_h), or none (nx_bh < 0): the loads are
   // still issued then (the wait counts stay the same) but fetch nothing
@@ -219,14 +223,14 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
     if (ip == 0) wait_vm<2 * PC + 2>(); else wait_vm<2 * PC + 2 + ST>();
     __builtin_amdgcn_s_barrier();
     load_q((j + 3) & 3);
-    v4i rq[PC], rk[PC];
+    // rotated values, rounded to the input type as the permuted tensors would hold them, kept in fp32
+    float fq[PC][8], fk[PC][8];
     float aq = 0.0000001f, ak = 0.0000001f;
 #pragma unroll
     for (int i = 0; i < PC; i++) {
-      rq[i] = own_piece(j & 3, i);
-      if (rope && src[i] >= p.n_text) rq[i] = rotate8<DT>(rq[i], cs[i], sn[i]);
+      rotate8_f32<DT>(own_piece(j & 3, i), rope && src[i] >= p.n_text, cs[i], sn[i], fq[i]);
 #pragma unroll
-      for (int e = 0; e < 8; e++) aq = fmaxf(aq, fabsf(elem16_to_f32<DT>(rq[i], e)));   // rows past the end are 0
+      for (int e = 0; e < 8; e++) aq = fmaxf(aq, fabsf(fq[i][e]));   // rows past the end are 0
     }
     aq = wave_max(aq);
     if (lane == 0) s_amax[0][wave] = aq;
@@ -243,11 +247,12 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
     }
 #pragma unroll
     for (int i = 0; i < PC; i++) {
-      rk[i] = own_piece((j + 1) & 3, i);
-      if (rope && src[i] >= p.n_text) rk[i] = rotate8<DT>(rk[i], cs[i], sn[i]);
-      if (src[i] >= 0) {  // rows past the end count as zero, whatever the mean
+      rotate8_f32<DT>(own_piece((j + 1) & 3, i), rope && src[i] >= p.n_text, cs[i], sn[i], fk[i]);
+      // the mean goes off here; rows past the end count as zero, whatever the mean
 #pragma unroll
-        for (int e = 0; e < 8; e++) ak = fmaxf(ak, fabsf(elem16_to_f32<DT>(rk[i], e) - mv[i % NV][e]));
+      for (int e = 0; e < 8; e++) {
+        fk[i][e] = src[i] >= 0 ? fk[i][e] - mv[i % NV][e] : 0.f;
+        ak = fmaxf(ak, fabsf(fk[i][e]));
       }
     }
     ak = wave_max(ak);
@@ -273,8 +278,8 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
         float yq[8], yk[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-          yq[e] = elem16_to_f32<DT>(rq[i], e) * inv_q;
-          yk[e] = (elem16_to_f32<DT>(rk[i], e) - mv[i % NV][e]) * inv_k;
+          yq[e] = fq[i][e] * inv_q;
+          yk[e] = fk[i][e] * inv_k;
         }
         const int o = (kb * 64 + 16 * wave + i * RPI + lane / LPR) * D + col[i % NV];
         __builtin_amdgcn_raw_buffer_store_b64(

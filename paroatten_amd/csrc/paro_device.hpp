@@ -88,6 +88,26 @@ __device__ __forceinline__ void* uniform_ptr(const void* ptr) {
   return reinterpret_cast<void*>(((unsigned long long)hi << 32) | lo);
 }
 
+// the same rotation (or none, ROT = false) with the result left in fp32: the values are those the
+// 16-bit result holds, so arithmetic on them equals arithmetic on a stored and reloaded tensor
+template <int DT>
+__device__ __forceinline__ void rotate8_f32(const v4i raw, bool rot, const float* cs, const float* sn, float* out) {
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const float x0 = lo16_to_f32<DT>((unsigned)raw[j]);
+    const float x1 = hi16_to_f32<DT>((unsigned)raw[j]);
+    out[2 * j] = x0;
+    out[2 * j + 1] = x1;
+    if (rot) {
+      const float o0 = __fsub_rn(__fmul_rn(x0, cs[2 * j]), __fmul_rn(x1, sn[2 * j]));
+      const float o1 = __fadd_rn(__fmul_rn(x1, cs[2 * j + 1]), __fmul_rn(x0, sn[2 * j + 1]));
+      const unsigned w = pack2_from_f32<DT>(o0, o1);
+      out[2 * j] = lo16_to_f32<DT>(w);
+      out[2 * j + 1] = hi16_to_f32<DT>(w);
+    }
+  }
+}
+
 // four values y (|y| <= 127.5, not yet rounded) -> four int8 = rint(y) packed in a word.  Adding
 // 1.5*2^23 rounds to the nearest integer, ties to even, exactly as rintf does (the sum lies in
 // [2^23, 2^24), where floats are the integers), and leaves the two's-complement byte in bits 0..7.
@@ -109,6 +129,7 @@ __device__ __forceinline__ unsigned pack4_rint_i8(float y0, float y1, float y2, 
 template <int DT, int D, int PITCH, bool SWZ = false>
 __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t* ob, const float* v_recp,
                                             const float* v_mean, int tok0, int N, int t) {
+  const bool full = tok0 + 64 <= N;    // uniform: only the last tile of a sequence checks its rows
 #pragma unroll
   for (int n = 0; n < D / 64; n++) {   // 4*D pieces, 256 threads
     const int c = t + 256 * n;
@@ -125,7 +146,7 @@ __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t*
         const int r = 32 * mt + 8 * g + 4 * (lane >> 5) + q;
         const int at = SWZ ? r * PITCH + ((((ch >> 3) ^ (((r >> 2) & 1) << 2)) << 3) | (ch & 7)) : r * PITCH + ch;
         const float x = F16x<DT>::to_f32(tile[at]);
-        f[q] = (tok0 + r < N) ? (x - mean) * rc : 0.f;
+        f[q] = (full || tok0 + r < N) ? (x - mean) * rc : 0.f;
       }
       int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
       p = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], p, true);
