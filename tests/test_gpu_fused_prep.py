@@ -135,6 +135,28 @@ def test_fused_prep_full_cogvideox_shape(dev):
     _same_v(got, ch[4], ch[5], ch[6])
 
 
+@pytest.mark.parametrize("B,H,same_order", [(36, 64, True), (5, 33, False)])
+def test_fused_prep_many_batch_head_pairs(dev, B, H, same_order):
+    """long lists of (batch, head) pairs per workgroup (2304 pairs of one order: the head split is
+    raised so that a workgroup's list fits) and pair counts that do not divide by the split."""
+    from paroatten_amd import permute as PM
+    from paroatten_amd import rope
+    D, grid, n_text = 64, (2, 4, 8), 5
+    N = n_text + 64
+    q, k, v = (t.to(dev) for t in synth.make_qkv(B, H, N, D, torch.bfloat16, seed=31))
+    if same_order:
+        orders = torch.full((H,), 4, dtype=torch.int32, device=dev)
+    else:
+        orders = PM.head_orders(synth.make_permute_plan(1, H, seed=32), 0, dev)
+    cos, sin = (t.to(dev) for t in rope.rope_table_cog(D, grid))
+    km = PM.rope_k_mean(k, grid, n_text, cos, sin)
+    got = PM.rope_permute_quant(q, k, v, orders, grid, n_text, cos, sin, km=km)
+    ch = _chain(dev, q, k, v, orders, grid, n_text, cos, sin, km)
+    assert torch.equal(got.q8, ch[0]) and torch.equal(got.q_scale, ch[1])
+    assert torch.equal(got.k8, ch[2]) and torch.equal(got.k_scale, ch[3])
+    _same_v(got, ch[4], ch[5], ch[6])
+
+
 def test_fused_prep_rejects_bad_arguments(dev):
     from paroatten_amd import permute as PM
     q = torch.zeros(1, 2, 128, 64, dtype=torch.float16, device=dev)
