@@ -301,7 +301,7 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
 // K mean over tokens AFTER the rotation (the permutation does not change a mean): partial sums per
 // 256-token chunk, then one workgroup per (batch, head) adds them in a fixed order.  A thread keeps
 // the table entries of its token piece while it walks over a group of (batch, head) pairs.
-constexpr int KM_GROUP = 8;
+constexpr int KM_GROUP = 4;   // measured: 4 beats 8 (too few workgroups at 40 heads) and 2 (tables re-read twice as often)
 template <int DT, int D>
 __global__ void __launch_bounds__(256) rope_k_sum_kernel(const unsigned short* __restrict__ k,
                                                          const float* __restrict__ cos_t,

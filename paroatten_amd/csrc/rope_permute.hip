@@ -114,10 +114,11 @@ static int launch_rp(const void* q_in, const void* k_in, const void* v_in, void*
                      int64_t os_b, int64_t os_h, int64_t os_n, hipStream_t st) {
   const int rows = 256 / (D / 8);
   const int BH = B * H;
-  // enough (batch, head) pairs per workgroup to amortise the rotary fragment, few enough that the
-  // launch still has several thousand workgroups
-  // (without tables there is nothing to amortise: one pair per workgroup, as a plain copy likes it)
-  int hpw = cos_t ? 16 : 1;
+  // (batch, head) pairs per workgroup: enough to amortise the rotary fragment (a table row is 8*D
+  // bytes per token, twice a token row), few enough that the launch has many short workgroups.
+  // Measured: D = 64 is fastest at 2..4 pairs (5.6-5.75 TB/s against 5.25 at 16), D = 128 at 16
+  // (5.5 against 5.4 at 4).  Without tables there is nothing to amortise: one pair per workgroup.
+  int hpw = cos_t ? (D == 64 ? 4 : 16) : 1;
   while (hpw > 1 && (int64_t)ceil_div(N, rows) * ceil_div(BH, hpw) < 3072) hpw >>= 1;
   dim3 grid(ceil_div(N, rows), ceil_div(BH, hpw)), block(256);
 #define PARO_RP(DTV, DV)                                                                                          \
