@@ -352,10 +352,16 @@ __global__ void __launch_bounds__(256) rope_k_sum_kernel(const unsigned short* _
   __shared__ float red[4][KM_GROUP][D];
 #pragma unroll
   for (int g = 0; g < KM_GROUP; g++) {
+    // lanes that share a column sit LPR apart
 #pragma unroll
-    for (int o = 32; o >= LPR; o >>= 1)
-#pragma unroll
-      for (int j = 0; j < 8; j++) s[g][j] += __shfl_xor(s[g][j], o, 64);
+    for (int j = 0; j < 8; j++) {
+      float a, b;
+      if constexpr (LPR == 8) s[g][j] += row_dpp<0x128>(s[g][j]);
+      with_lane_xor16(s[g][j], a, b);
+      s[g][j] = a + b;
+      with_lane_xor32(s[g][j], a, b);
+      s[g][j] = a + b;
+    }
     if (lane < LPR) {
 #pragma unroll
       for (int j = 0; j < 8; j++) red[wave][g][col + j] = s[g][j];

@@ -64,10 +64,35 @@ template <> struct F16x<PARO_DTYPE_BF16> {
   }
 };
 
+// ---- cross-lane exchange without the LDS crossbar ----------------------------------------------
+// value of another lane of the same 16-lane row: DPP control 0xB1 = lane ^ 1, 0x4E = lane ^ 2,
+// 0x124 / 0x128 = four / eight lanes further round the row
+template <int CTRL> __device__ __forceinline__ float row_dpp(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+// {own value, value of lane ^ 16} resp. {.., lane ^ 32} in some order: the swaps exchange the odd
+// rows (upper half) of their first operand with the even rows (lower half) of their second
+__device__ __forceinline__ void with_lane_xor16(float x, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+__device__ __forceinline__ void with_lane_xor32(float x, float& a, float& b) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  a = __uint_as_float(r[0]);
+  b = __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fmaxf(v, row_dpp<0xB1>(v));
+  v = fmaxf(v, row_dpp<0x4E>(v));
+  v = fmaxf(v, row_dpp<0x124>(v));
+  v = fmaxf(v, row_dpp<0x128>(v));
+  float a, b;
+  with_lane_xor16(v, a, b);
+  v = fmaxf(a, b);
+  with_lane_xor32(v, a, b);
+  return fmaxf(a, b);
 }
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }

@@ -47,15 +47,21 @@ __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __re
       }
     }
   }
-  // lanes that share a column sit LPR apart
+  // lanes that share a column sit LPR apart: 8 lanes round the row (D = 64 only), then lane ^ 16, ^ 32
 #pragma unroll
-  for (int o = 32; o >= LPR; o >>= 1) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      s[j] += __shfl_xor(s[j], o, 64);
-      mn[j] = fminf(mn[j], __shfl_xor(mn[j], o, 64));
-      mx[j] = fmaxf(mx[j], __shfl_xor(mx[j], o, 64));
+  for (int j = 0; j < 8; j++) {
+    float a, b;
+    if constexpr (LPR == 8) {
+      s[j] += row_dpp<0x128>(s[j]);
+      mn[j] = fminf(mn[j], row_dpp<0x128>(mn[j]));
+      mx[j] = fmaxf(mx[j], row_dpp<0x128>(mx[j]));
     }
+    with_lane_xor16(s[j], a, b);  s[j] = a + b;
+    with_lane_xor16(mn[j], a, b); mn[j] = fminf(a, b);
+    with_lane_xor16(mx[j], a, b); mx[j] = fmaxf(a, b);
+    with_lane_xor32(s[j], a, b);  s[j] = a + b;
+    with_lane_xor32(mn[j], a, b); mn[j] = fminf(a, b);
+    with_lane_xor32(mx[j], a, b); mx[j] = fmaxf(a, b);
   }
   __shared__ float red[4][3][D];
   if (lane < LPR) {
