@@ -8,6 +8,13 @@
  * Return value: PARO_OK or a negative PARO_ERR_* code; paro_last_error() gives the message
  * of the last failure on the calling thread.
  *
+ * Size limits, checked by every entry point they apply to (PARO_ERR_RUNTIME beyond them): batch and
+ * head counts up to 65535 each (they are launch-grid dimensions; the permutation and preparation
+ * entry points need batch * heads <= 65535); kernels that address one (batch, head) slice through a
+ * 32-bit buffer descriptor (attention: K8 / V8; one-pass preparation: q, k, v, q8, k8) need that slice,
+ * (N - 1) * token stride + D elements, below 2 GiB; the attention kernel keeps the list of kept key
+ * blocks in the local data share, which bounds kv_len at about 1.4 million tokens.
+ *
  * Each entry point names the interface of the reference (jamescsq47/PAROAtten) it stands in
  * for, as file:line relative to the reference tree.
  */
