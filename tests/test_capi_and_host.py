@@ -156,3 +156,34 @@ def test_new_entry_points_validate_without_gpu():
     assert rc == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
     rc = lib.paro_rope_k_mean(p, 0, p, None, p, p, 1 << 20, 1, 1, 128, 64, 0, 2, 8, 8, 8192, 8192, 64, 64, 64, None)
     assert rc == L.PARO_ERR_RUNTIME and b"cos and sin" in lib.paro_last_error()
+
+
+def test_size_limits_are_rejected_without_gpu():
+    """batch * heads beyond the launch-grid range, slices beyond the 32-bit buffer offsets and key
+    lists beyond the local data share come back as errors, not launches"""
+    import paroatten_amd._lib as L
+    lib = L.load()
+    buf = ctypes.create_string_buffer(8192)
+    p = ctypes.c_void_p((ctypes.addressof(buf) + 255) & ~255)
+    N, D = 128, 64
+    rc = lib.paro_rope_permute_fwd(p, None, None, p, None, None, 0, None, None, p, 1024, 64, N, D, 0, 2, 8, 8,
+                                   64 * N * D, N * D, D, 64 * N * D, N * D, D, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"exceeds 65535" in lib.paro_last_error()
+    rc = lib.paro_quant_int8(p, 0, None, p, p, 1, 70000, N, D, 0, N * D, D, 0, 0, 0, N * D, D, 0, 2, 64, 2, 0, 0.0, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"exceeds 65535" in lib.paro_last_error()
+    # one-pass preparation: a token stride that puts the last row of a head 2 GiB away
+    big = 1 << 24
+    rc = lib.paro_rope_permute_quant_fwd(p, p, p, 0, None, None, p, None, p, p, p, p, p, p, p, p, 1 << 20,
+                                         1, 1, N, D, 0, 2, 8, 8, 0, 0, big, N * D, N * D, D, N * D, N * D, D,
+                                         0, 0, 1, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"2 GiB" in lib.paro_last_error()
+    # attention: 30 million keys = 468 750 blocks, far more than the 65 535 a block index can hold
+    Nk = 30_000_000
+    rc = lib.paro_attn_sparse_fwd(p, p, p, p, p, p, p, p, 0, p, 0, None, None, 1, 1, 1, 64, Nk, D,
+                                  64 * D, 64 * D, D, Nk * D, Nk * D, D, 64 * D, 64 * D, D, 0.125, 0, 0, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"exceeds 65535 blocks" in lib.paro_last_error()
+    # 2 million keys fit the block index but not the list in the local data share
+    Nk = 2_000_000
+    rc = lib.paro_attn_sparse_fwd(p, p, p, p, p, p, p, p, 0, p, 0, None, None, 1, 1, 1, 64, Nk, D,
+                                  64 * D, 64 * D, D, Nk * D, Nk * D, D, 64 * D, 64 * D, D, 0.125, 0, 0, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"local data share" in lib.paro_last_error()
