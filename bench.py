@@ -201,6 +201,12 @@ def main():
         timed("permute_inverse_o", lambda: PM.permute_inverse(out, orders, wl.grid, wl.n_text), 2 * el * 2)
         # the same work as separate kernels (what the fused pass replaces)
         timed("rope_permute_qkv", lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), 3 * 2 * el * 2)
+        if wl.dtype != torch.bfloat16:
+            # the RoPE + permutation configuration of the benchmark list is bfloat16, q and k only
+            qb, kb = q.to(torch.bfloat16), k.to(torch.bfloat16)
+            timed("rope_permute_qk_bf16", lambda: PM.rope_permute(qb, kb, None, orders, wl.grid, wl.n_text, cos, sin),
+                  2 * 2 * el * 2)
+            del qb, kb
         timed("quant_int8_qk", lambda: Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64), 2 * el * 3)
         timed("v_fp8_pack", lambda: Q.per_channel_fp8(vp), el * 5)
         # plain device copy of one tensor: what this box sustains for the simplest read+write
