@@ -299,7 +299,7 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
 }
 
 // K mean over tokens AFTER the rotation (the permutation does not change a mean): partial sums per
-// 256-token chunk, then one workgroup per (batch, head) adds them in a fixed order.  A thread keeps
+// K_CHUNK-token chunk, then one workgroup per (batch, head) adds them in a fixed order.  A thread keeps
 // the table entries of its token piece while it walks over a group of (batch, head) pairs.
 constexpr int KM_GROUP = 4;   // measured: 4 beats 8 (too few workgroups at 40 heads) and 2 (tables re-read twice as often)
 template <int DT, int D>
@@ -320,8 +320,8 @@ __global__ void __launch_bounds__(256) rope_k_sum_kernel(const unsigned short* _
   for (int g = 0; g < KM_GROUP; g++)
 #pragma unroll
     for (int j = 0; j < 8; j++) s[g][j] = 0.f;
-  for (int r = t / LPR; r < V_CHUNK; r += ROWS) {
-    const int tok = chunk * V_CHUNK + r;
+  for (int r = t / LPR; r < K_CHUNK; r += ROWS) {
+    const int tok = chunk * K_CHUNK + r;
     if (tok >= N) break;
     const bool rot = cos_t != nullptr && tok >= n_text;
     float cs[8], sn[8];
@@ -425,8 +425,10 @@ static int check_prep(const char* fn, int dtype, int B, int H, int N, int D, int
 }  // namespace paro
 
 extern "C" int64_t paro_prep_workspace_bytes(int B, int H, int N, int D) {
-  // per-chunk partials of the V statistics (sum, min, max); the K mean needs a third of that
-  return paro_v_fp8_partial_floats(B, H, N, D) * 4;
+  // per-chunk partials of the V statistics (sum, min, max) or of the K mean (sums), whichever is larger
+  const int64_t v_part = paro_v_fp8_partial_floats(B, H, N, D);
+  const int64_t k_part = (int64_t)B * H * paro::ceil_div(N, paro::K_CHUNK) * D;
+  return (v_part > k_part ? v_part : k_part) * 4;
 }
 
 extern "C" int paro_rope_k_mean(const void* k, int dtype, const float* cos, const float* sin, void* k_mean,
@@ -441,7 +443,7 @@ extern "C" int paro_rope_k_mean(const void* k, int dtype, const float* cos, cons
   PARO_CHECK(((uintptr_t)k % 16) == 0 && ((uintptr_t)cos % 16) == 0 && ((uintptr_t)sin % 16) == 0 &&
                  ((uintptr_t)workspace % 16) == 0,
              PARO_ERR_RUNTIME, "paro_rope_k_mean: tensors must be 16-byte aligned");
-  const int n_chunks = ceil_div(N, V_CHUNK);
+  const int n_chunks = ceil_div(N, K_CHUNK);
   PARO_CHECK(workspace_bytes >= (int64_t)B * H * n_chunks * D * 4, PARO_ERR_RUNTIME,
              "paro_rope_k_mean: workspace of %lld bytes is too small", (long long)workspace_bytes);
   hipStream_t st = (hipStream_t)stream;

@@ -4,7 +4,11 @@
 
 namespace paro {
 
-constexpr int V_CHUNK = 256;  // tokens per chunk of the per-channel V statistics
+// tokens per workgroup of the two statistics passes.  Measured: the V statistics (three values per
+// channel to reduce and write) want long chunks, 1024 beats 256 by 7 %; the K mean, launched per group
+// of heads, runs out of workgroups beyond 256.
+constexpr int V_CHUNK = 1024;  // per-channel V statistics
+constexpr int K_CHUNK = 256;   // rotated K mean
 
 // strides of the (f,h,w) coordinates in the permuted order `order`
 // (0 FHW, 1 FWH, 2 HWF, 3 HFW, 4 WHF, 5 WFH).  Written as selects: a switch that assigns through the

@@ -3,7 +3,7 @@
 // tiles straight from HBM to LDS and reads each A operand as one contiguous 16-byte piece per lane.
 //
 // Three launches, all HBM-bound and deterministic (no float atomics):
-//   v_stats    : per 256-token chunk, per channel: sum, min, max          (reads V once)
+//   v_stats    : per V_CHUNK-token chunk, per channel: sum, min, max      (reads V once)
 //   v_finalize : per (b,h,channel): mean = sum/N, amax = max(max-mean, mean-min), scale = amax/448,
 //                recp = 448/amax
 //   v_pack     : per 64-token tile: (v-mean)*recp -> e4m3, fragment order  (reads V once more)
