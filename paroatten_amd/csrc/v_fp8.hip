@@ -32,19 +32,31 @@ __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __re
     mn[j] = INFINITY;
     mx[j] = -INFINITY;
   }
-#pragma unroll 4
-  for (int r = t / LPR; r < V_CHUNK; r += ROWS) {
-    const int tok = chunk * V_CHUNK + r;
-    if (tok < N) {
-      const v4i raw = *reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n);
+  auto take = [&](const v4i raw) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) {
-        const unsigned w = (unsigned)raw[j >> 1];
-        const float f = F16x<DT>::to_f32((unsigned short)((j & 1) ? (w >> 16) : (w & 0xffffu)));
-        s[j] += f;
-        mn[j] = fminf(mn[j], f);
-        mx[j] = fmaxf(mx[j], f);
-      }
+    for (int j = 0; j < 8; j++) {
+      const float f = elem16_to_f32<DT>(raw, j);
+      s[j] += f;
+      mn[j] = fminf(mn[j], f);
+      mx[j] = fmaxf(mx[j], f);
+    }
+  };
+  const int tok0 = chunk * V_CHUNK + t / LPR;
+  if (chunk * V_CHUNK + V_CHUNK <= N) {
+    // full chunk (uniform): batches of VS_BATCH independent loads, then the arithmetic
+    constexpr int VS_BATCH = 8;
+    for (int r = 0; r < V_CHUNK; r += ROWS * VS_BATCH) {
+      v4i raw[VS_BATCH];
+#pragma unroll
+      for (int u = 0; u < VS_BATCH; u++)
+        raw[u] = *reinterpret_cast<const v4i*>(vb + (int64_t)(tok0 + r + u * ROWS) * vs_n);
+#pragma unroll
+      for (int u = 0; u < VS_BATCH; u++) take(raw[u]);
+    }
+  } else {
+    for (int r = 0; r < V_CHUNK; r += ROWS) {
+      const int tok = tok0 + r;
+      if (tok < N) take(*reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n));
     }
   }
   // lanes that share a column sit LPR apart: 8 lanes round the row (D = 64 only), then lane ^ 16, ^ 32
