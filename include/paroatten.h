@@ -126,7 +126,8 @@ int paro_attn_sparse_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
  * below for order orders[head] (rows below n_text stay in place).  Stands in for the attention call
  * followed by permute_attn_out (paroattention/cogvideox.py:216-227; wan.py:276,300): with
  * out strides of a [B,N,H,D] buffer the result is token-major, ready for the output projection.
- * Requires Nq == n_text + F*Hh*W.  orders: int32 [H] on the device. */
+ * Requires Nq == n_text + F*Hh*W.  orders: int32 [H] on the device.  lse, if given, stays in the
+ * order of the q-rows (the permuted order): only `out` is stored through the inverse permutation. */
 int paro_attn_sparse_unpermute_fwd(const int8_t* q8, const int8_t* k8, const uint8_t* v8,
                                    const float* q_scale, const float* k_scale,
                                    const float* v_scale, const float* v_mean,
