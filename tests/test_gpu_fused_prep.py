@@ -193,6 +193,14 @@ def test_attention_with_folded_inverse_permutation(dev, D, grid, n_text, dtype):
     qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, token_major.transpose(1, 2),
                                 ops.q_scale, ops.k_scale, D ** -0.5, mask, unpermute=(orders, grid, n_text))
     assert torch.equal(token_major.transpose(1, 2), want)
+    # with the log-sum-exp (exact exponentials): lse stays in q-row order, the output is unpermuted
+    lse_p = qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, plain, ops.q_scale,
+                                        ops.k_scale, D ** -0.5, mask, return_lse=1)
+    lse_u = qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, token_major.transpose(1, 2),
+                                        ops.q_scale, ops.k_scale, D ** -0.5, mask, return_lse=1,
+                                        unpermute=(orders, grid, n_text))
+    assert torch.equal(lse_p, lse_u)
+    assert torch.equal(token_major.transpose(1, 2), PM.permute_inverse(plain, orders, grid, n_text))
     with pytest.raises(RuntimeError):
         qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, plain, ops.q_scale, ops.k_scale,
                                     D ** -0.5, mask, unpermute=(orders, (grid[0], grid[1], grid[2] + 1), n_text))
