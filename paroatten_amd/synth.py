@@ -94,6 +94,18 @@ def make_block_mask(H, nb, density, seed=0, band=2, device="cpu"):
     return mask.reshape(H, nb, nb)
 
 
+def make_window_mask(H, nb, density, device="cpu"):
+    """bool [H, nb, nb]: every q-block keeps one contiguous run of round(density * nb) k-blocks
+    centred on the diagonal (clipped at the ends): the shape the masks of a permuted head have, as
+    opposed to the uniformly scattered extra blocks of make_block_mask."""
+    w = max(1, min(nb, int(round(density * nb))))
+    i = torch.arange(nb, device=device)
+    lo = (i - w // 2).clamp(0, nb - w)
+    j = i[None, :]
+    m = (j >= lo[:, None]) & (j < lo[:, None] + w)
+    return m[None].expand(H, nb, nb).contiguous()
+
+
 def make_permute_plan(n_layers, H, seed=0):
     """{'permute': int64 [L,H] in 0..5, 'empty': bool [L,H]} (all heads non-empty)."""
     g = torch.Generator(device="cpu").manual_seed(seed)

@@ -118,6 +118,9 @@ def test_mask_generator_contract():
         i = torch.arange(nb)
         assert m[:, i, i].all() and m[:, i[:-2], i[:-2] + 2].all() and m[:, i[2:], i[2:] - 2].all()
     assert torch.equal(synth.make_block_mask(2, 16, 0.4, seed=5), synth.make_block_mask(2, 16, 0.4, seed=5))
+    w = synth.make_window_mask(2, 40, 0.2)
+    assert w.shape == (2, 40, 40) and (w.sum(dim=2) == 8).all() and w[:, torch.arange(40), torch.arange(40)].all()
+    assert ((w[0].int().diff(dim=1) != 0).sum(dim=1) <= 2).all()      # one contiguous run per row
     plan = synth.make_permute_plan(4, 48, seed=0)
     assert plan["permute"].shape == (4, 48) and int(plan["permute"].min()) >= 0 and int(plan["permute"].max()) <= 5
 
