@@ -77,6 +77,10 @@ int paro_quant_int8(const void* x, int dtype, const void* mean, int8_t* out, flo
  *
  * v [B,Hkv,N,D] 16-bit.  v_mean, v_scale: fp32 [B,Hkv,D] (contiguous).  v8: paro_v_fp8_bytes().
  *   mean = sum_n v / N (0 if !smooth) ; scale = max|v - mean| / 448 ; v8 = e4m3_rne((v-mean)/scale)
+ *   v_mean = mean + sum_n (v - mean - scale * v8) / N   (if smooth)
+ * i.e. v_mean is the offset the attention epilogue adds back: the channel mean plus the mean rounding
+ * residual of the channel's codes (a few 1e-4 of max|v|; rounding 16-bit inputs to e4m3 is not unbiased,
+ * and a per-channel bias does not average out over the keys of a row the way rounding noise does).
  * Tile order: v8[((b*Hkv+h)*nb + kb)*64*D + ((dt*2 + mt)*64 + lane)*16 + r] holds token
  * kb*64 + 32*mt + 8*(r/4) + 4*(lane/32) + r%4, channel 32*dt + lane%32 (tokens >= N are 0).
  * partial: fp32 work buffer of paro_v_fp8_partial_floats() floats.

@@ -50,6 +50,7 @@ struct PrepParams {
   float* k_scale;
   uint8_t* v8;
   const float* v_stats;  // per (batch, head): D reciprocal scales, then D means, at v_recp_offset
+  float* v_resid;        // rounding residual sums of the V codes, [B*H][nb][2][D] (nullptr: not wanted)
   int BH, H, N, nb, n_text, F, Hh, W, head_split;
   int64_t qs_b, qs_h, qs_n, ks_b, ks_h, ks_n, vs_b, vs_h, vs_n, ms_b, ms_h;
 };
@@ -87,8 +88,9 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
   constexpr int PC = 16 / RPI;          // pieces per lane and tile: a wave owns 16 rows of the block
   constexpr int NV = D == 128 ? 2 : 1;  // distinct channel offsets among a lane's pieces
   // vector-memory operations one wave issues per pair: PC per tile, two more with the K tile (mean
-  // row, V statistics row), and ST stores that are issued unconditionally (q8, k8: PC each, v8: D/64)
-  constexpr int ST = 2 * PC + D / 64;
+  // row, V statistics row), and ST stores that are issued unconditionally (q8, k8: PC each, v8 and its
+  // residual sums: D/64 each)
+  constexpr int ST = 2 * PC + 2 * (D / 64);
   constexpr int OOB = 0x7ffffff0;       // offset beyond any descriptor range
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -290,8 +292,20 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
     }
     // V tile -> e4m3 fragments
     const float* st = reinterpret_cast<const float*>(smem + L::ST_OFF + par * 1024);
+    float rs[D / 64];
     pack_v_tile<DT, D, D, true>(reinterpret_cast<const unsigned short*>(smem + ((j + 2) & 3) * L::TILE),
-                                p.v8 + ((int64_t)bh * p.nb + kb) * (int64_t)(64 * D), st, st + D, kb * 64, p.N, t);
+                                p.v8 + ((int64_t)bh * p.nb + kb) * (int64_t)(64 * D), st, st + D, kb * 64, p.N, t, rs);
+    {
+      // lanes 0..31 hold the sums of row tile wave%2, channels 32*(wave/2 + 2n) + lane; the store is issued
+      // by every wave whether wanted or not (a descriptor of 0 bytes drops it), so the wait counts hold
+      const __amdgpu_buffer_rsrc_t rr =
+          raw_buffer(p.v_resid ? p.v_resid + ((int64_t)bh * p.nb + kb) * (2 * D) : p.q_scale, p.v_resid ? 2 * D * 4 : 0);
+#pragma unroll
+      for (int n = 0; n < D / 64; n++)
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(rs[n]), rr,
+                                              lane < 32 ? ((wave & 1) * D + 32 * ((wave >> 1) + 2 * n) + lane) * 4 : OOB,
+                                              0, 0);
+    }
     j = (j + 3) & 3;
   }
   // the loads issued for the pair after the last one fetch nothing, but they do write LDS
@@ -519,6 +533,7 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
   p.q = (const unsigned short*)q; p.k = (const unsigned short*)k; p.v = (const unsigned short*)v;
   p.cos_t = cos; p.sin_t = sin; p.orders = (const int*)orders; p.k_mean = (const unsigned short*)k_mean;
   p.q8 = q8; p.q_scale = q_scale; p.k8 = k8; p.k_scale = k_scale; p.v8 = v8; p.v_stats = (const float*)workspace;
+  p.v_resid = smooth_v ? (float*)workspace + v_resid_offset((int64_t)B * H, ceil_div(N, V_CHUNK), D) : nullptr;
   p.BH = B * H; p.H = H; p.N = N; p.nb = nb; p.n_text = n_text; p.F = F; p.Hh = Hh; p.W = W; p.head_split = head_split;
   p.qs_b = q_stride_b; p.qs_h = q_stride_h; p.qs_n = q_stride_n;
   p.ks_b = k_stride_b; p.ks_h = k_stride_h; p.ks_n = k_stride_n;
@@ -535,5 +550,6 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
 #undef PARO_PREP
   if (rc) return rc;
   PARO_HIP(hipGetLastError());
+  if (p.v_resid) return v_fp8_add_residual(p.v_resid, v_scale, v_mean, B, H, N, D, st);
   return PARO_OK;
 }

@@ -130,9 +130,13 @@ __device__ __forceinline__ unsigned pack4_rint_i8(float y0, float y1, float y2, 
 // (0 for a constant channel), as MeanScaleKernel of the reference forms it
 // (csrc/fused/fused.cu:399,414).  256 threads.  SWZ: rows are unpadded (PITCH = D) and 16-byte chunk c
 // of row r sits at chunk position c ^ 4*((r >> 2) & 1).
+// resid[n] (n < D/64): the rounding residual sum over the 32 tokens of row tile mt = wave%2 of
+// (v - mean)*recp - e4m3(that), for channel 32*(wave/2 + 2n) + lane%32, the same value in lanes l and
+// l^32.  Its mean over all tokens, times the scale, is what the codes of a channel are off by on
+// average: the attention epilogue adds it back together with the channel mean.
 template <int DT, int D, int PITCH, bool SWZ = false>
 __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t* ob, const float* v_recp,
-                                            const float* v_mean, int tok0, int N, int t) {
+                                            const float* v_mean, int tok0, int N, int t, float* resid) {
   const bool full = tok0 + 64 <= N;    // uniform: only the last tile of a sequence checks its rows
 #pragma unroll
   for (int n = 0; n < D / 64; n++) {   // 4*D pieces, 256 threads
@@ -142,6 +146,7 @@ __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t*
     const float mean = v_mean ? v_mean[ch] : 0.f;
     const float rc = v_recp[ch];
     int w[4];
+    float es = 0.f;
 #pragma unroll
     for (int g = 0; g < 4; g++) {
       float f[4];
@@ -155,10 +160,18 @@ __device__ __forceinline__ void pack_v_tile(const unsigned short* tile, uint8_t*
       int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
       p = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], p, true);
       w[g] = p;
+      es += ((f[0] - __builtin_amdgcn_cvt_f32_fp8(p, 0)) + (f[1] - __builtin_amdgcn_cvt_f32_fp8(p, 1))) +
+            ((f[2] - __builtin_amdgcn_cvt_f32_fp8(p, 2)) + (f[3] - __builtin_amdgcn_cvt_f32_fp8(p, 3)));
     }
     __builtin_nontemporal_store(v4i{w[0], w[1], w[2], w[3]}, reinterpret_cast<v4i*>(ob + (int64_t)c * 16));
+    float a, b;
+    with_lane_xor32(es, a, b);
+    resid[n] = a + b;
   }
 }
+
+// residual sums of pack_v_tile: [B*Hkv][nb][2 row tiles][D] floats behind the statistics partials
+__host__ __device__ inline int64_t v_resid_offset(int64_t BH, int n_chunks, int D) { return BH * n_chunks * 3 * D; }
 
 // where v_fp8_stats leaves recp[b,h,:] inside the partial-sum workspace
 __host__ __device__ inline int64_t v_recp_offset(int64_t bh, int n_chunks, int D) { return bh * n_chunks * 3 * D; }
@@ -168,5 +181,8 @@ __host__ __device__ inline int64_t v_recp_offset(int64_t bh, int n_chunks, int D
 // two launches on `st` (defined in v_fp8.hip)
 int v_fp8_stats(const void* v, int dtype, float* v_scale, float* v_mean, float* partial, int B, int Hkv, int N,
                 int D, int64_t vs_b, int64_t vs_h, int64_t vs_n, int smooth, hipStream_t st);
+// v_mean[b,h,ch] += v_scale[b,h,ch] * (sum of the channel's residual sums) / N, in a fixed order (one launch)
+int v_fp8_add_residual(const float* resid, const float* v_scale, float* v_mean, int B, int Hkv, int N, int D,
+                       hipStream_t st);
 
 }  // namespace paro

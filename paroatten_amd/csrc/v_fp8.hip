@@ -6,7 +6,13 @@
 //   v_stats    : per V_CHUNK-token chunk, per channel: sum, min, max      (reads V once)
 //   v_finalize : per (b,h,channel): mean = sum/N, amax = max(max-mean, mean-min), scale = amax/448,
 //                recp = 448/amax
-//   v_pack     : per 64-token tile: (v-mean)*recp -> e4m3, fragment order  (reads V once more)
+//   v_pack     : per 64-token tile: (v-mean)*recp -> e4m3, fragment order  (reads V once more), and the
+//                tile's rounding residual sums per channel
+//   v_residual : per (b,h,channel): v_mean += scale * (sum of residuals) / N
+// The last step removes the mean error of the codes: rounding (v-mean)/scale to e4m3 is unbiased only if
+// the values are spread evenly over the rounding cells, and 16-bit inputs (bfloat16 above all, with its 8
+// significant bits) are a lattice that is not; what is left, ~3e-4 of max|v| per channel, does not
+// average out over the keys of an attention row, whereas the rounding noise does.
 // max|v-mean| over tokens equals max(max-mean, mean-min) exactly because fp32 subtraction is
 // monotonic, so no second reduction pass is needed.
 // Arithmetic follows MeanScaleKernel of the reference (csrc/fused/fused.cu:316-427) except that the
@@ -137,7 +143,8 @@ template <int DT, int D>
 __global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __restrict__ v,
                                                      uint8_t* __restrict__ v8,
                                                      const float* __restrict__ v_recp,
-                                                     const float* __restrict__ v_mean, int N, int nb, int n_chunks,
+                                                     const float* __restrict__ v_mean, float* __restrict__ resid,
+                                                     int N, int nb, int n_chunks,
                                                      int64_t vs_b, int64_t vs_h, int64_t vs_n) {
   constexpr int LPR = D / 8;
   constexpr int ROWS = 256 / LPR;
@@ -156,8 +163,47 @@ __global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __res
     *reinterpret_cast<v4i*>(&tile[r * PITCH + col]) = raw;
   }
   __syncthreads();
+  float rs[D / 64];
   pack_v_tile<DT, D, PITCH>(tile, v8 + (bh * nb + kb) * (int64_t)(64 * D), v_recp + v_recp_offset(bh, n_chunks, D),
-                            v_mean ? v_mean + bh * D : nullptr, kb * 64, N, t);
+                            v_mean ? v_mean + bh * D : nullptr, kb * 64, N, t, rs);
+  if (resid != nullptr && (t & 63) < 32) {
+    const int wave = t >> 6;
+#pragma unroll
+    for (int n = 0; n < D / 64; n++)
+      resid[((bh * nb + kb) * 2 + (wave & 1)) * D + 32 * ((wave >> 1) + 2 * n) + (t & 31)] = rs[n];
+  }
+}
+
+// v_mean += v_scale * (sum over tiles and row tiles of the residual sums) / N; 1024 / D slices of the
+// tile range per channel, combined through LDS in a fixed order
+template <int D>
+__global__ void __launch_bounds__(1024) v_residual_kernel(const float* __restrict__ resid,
+                                                          const float* __restrict__ v_scale,
+                                                          float* __restrict__ v_mean, int N, int n_rows) {
+  constexpr int SL = 1024 / D;
+  __shared__ float red[SL][D];
+  const int ch = threadIdx.x % D, sl = threadIdx.x / D;
+  const int64_t bh = blockIdx.x;
+  const float* p = resid + bh * n_rows * D;
+  float s = 0.f;
+  for (int c = sl; c < n_rows; c += SL) s += p[(int64_t)c * D + ch];
+  red[sl][ch] = s;
+  __syncthreads();
+  if (sl == 0) {
+    for (int i = 1; i < SL; i++) s += red[i][ch];
+    v_mean[bh * D + ch] += v_scale[bh * D + ch] * (s / (float)N);
+  }
+}
+
+int v_fp8_add_residual(const float* resid, const float* v_scale, float* v_mean, int B, int Hkv, int N, int D,
+                       hipStream_t st) {
+  const int n_rows = ceil_div(N, 64) * 2;
+  if (D == 64)
+    hipLaunchKernelGGL((v_residual_kernel<64>), dim3(B * Hkv), dim3(1024), 0, st, resid, v_scale, v_mean, N, n_rows);
+  else
+    hipLaunchKernelGGL((v_residual_kernel<128>), dim3(B * Hkv), dim3(1024), 0, st, resid, v_scale, v_mean, N, n_rows);
+  PARO_HIP(hipGetLastError());
+  return PARO_OK;
 }
 
 template <int DT, int D>
@@ -184,12 +230,15 @@ int v_fp8_stats(const void* v, int dtype, float* v_scale, float* v_mean, float* 
 }
 
 template <int DT, int D>
-static int run_v_pack(const void* v, uint8_t* v8, const float* v_recp, const float* v_mean, int B, int Hkv, int N,
-                      int64_t vs_b, int64_t vs_h, int64_t vs_n, hipStream_t st) {
-  const int nb = ceil_div(N, 64);
+static int run_v_pack(const void* v, uint8_t* v8, float* partial, float* v_scale, float* v_mean, int B, int Hkv,
+                      int N, int64_t vs_b, int64_t vs_h, int64_t vs_n, hipStream_t st) {
+  const int nb = ceil_div(N, 64), n_chunks = ceil_div(N, V_CHUNK);
+  // without smoothing there is no mean to correct
+  float* resid = v_mean ? partial + v_resid_offset((int64_t)B * Hkv, n_chunks, D) : nullptr;
   hipLaunchKernelGGL((v_pack_kernel<DT, D>), dim3(nb, Hkv, B), dim3(256), 0, st, (const unsigned short*)v, v8,
-                     v_recp, v_mean, N, nb, ceil_div(N, V_CHUNK), vs_b, vs_h, vs_n);
+                     partial, v_mean, resid, N, nb, n_chunks, vs_b, vs_h, vs_n);
   PARO_HIP(hipGetLastError());
+  if (resid) return v_fp8_add_residual(resid, v_scale, v_mean, B, Hkv, N, D, st);
   return PARO_OK;
 }
 
@@ -231,7 +280,8 @@ extern "C" int64_t paro_v_fp8_bytes(int B, int Hkv, int N, int D) {
   return (int64_t)B * Hkv * paro::ceil_div(N, 64) * 64 * D;
 }
 extern "C" int64_t paro_v_fp8_partial_floats(int B, int Hkv, int N, int D) {
-  return (int64_t)B * Hkv * paro::ceil_div(N, paro::V_CHUNK) * 3 * D;
+  // statistics partials (sum, min, max per chunk and channel), then the residual sums per row tile
+  return (int64_t)B * Hkv * ((int64_t)paro::ceil_div(N, paro::V_CHUNK) * 3 + (int64_t)paro::ceil_div(N, 64) * 2) * D;
 }
 
 extern "C" int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_scale, float* v_mean,
@@ -253,13 +303,13 @@ extern "C" int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_s
   if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, partial, B, Hkv, N, D, v_stride_b, v_stride_h, v_stride_n,
                            smooth, st))
     return rc;
-  const float* mean = smooth ? v_mean : nullptr;
+  float* mean = smooth ? v_mean : nullptr;
   if (dtype == PARO_DTYPE_F16) {
-    if (D == 64) return run_v_pack<PARO_DTYPE_F16, 64>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
-    return run_v_pack<PARO_DTYPE_F16, 128>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
+    if (D == 64) return run_v_pack<PARO_DTYPE_F16, 64>(v, v8, partial, v_scale, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
+    return run_v_pack<PARO_DTYPE_F16, 128>(v, v8, partial, v_scale, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
   }
-  if (D == 64) return run_v_pack<PARO_DTYPE_BF16, 64>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
-  return run_v_pack<PARO_DTYPE_BF16, 128>(v, v8, partial, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
+  if (D == 64) return run_v_pack<PARO_DTYPE_BF16, 64>(v, v8, partial, v_scale, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
+  return run_v_pack<PARO_DTYPE_BF16, 128>(v, v8, partial, v_scale, mean, B, Hkv, N, v_stride_b, v_stride_h, v_stride_n, st);
 }
 
 extern "C" int paro_sub_mean(const void* v, int dtype, const void* mean, void* out_f16, int B, int H, int N,

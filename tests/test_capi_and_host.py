@@ -36,8 +36,9 @@ def test_size_queries_need_no_gpu():
     import paroatten_amd._lib as L
     lib = L.load()
     assert lib.paro_v_fp8_bytes(2, 48, 17776, 64) == 2 * 48 * 278 * 64 * 64
-    assert lib.paro_v_fp8_partial_floats(1, 1, 1024, 64) == 3 * 64            # one chunk of 1024 tokens
-    assert lib.paro_v_fp8_partial_floats(1, 1, 1025, 128) == 2 * 3 * 128
+    # statistics: 3 values per chunk of 1024 tokens and channel; residual sums: 2 per 64-token tile
+    assert lib.paro_v_fp8_partial_floats(1, 1, 1024, 64) == (3 + 16 * 2) * 64
+    assert lib.paro_v_fp8_partial_floats(1, 1, 1025, 128) == (2 * 3 + 17 * 2) * 128
     ws = lib.paro_attn_workspace_bytes(2, 48, 17776, 64)
     assert ws >= lib.paro_v_fp8_bytes(2, 48, 17776, 64) and ws % 256 == 0
 
@@ -138,7 +139,8 @@ def test_new_entry_points_validate_without_gpu():
     p = ctypes.c_void_p((ctypes.addressof(buf) + 255) & ~255)
     odd = ctypes.c_void_p(p.value + 4)
     assert lib.paro_mask_unpack(odd, p, 64, None) == L.PARO_ERR_RUNTIME and b"aligned" in lib.paro_last_error()
-    assert lib.paro_prep_workspace_bytes(2, 48, 17776, 64) == 2 * 48 * 70 * 64 * 4    # K-mean partials: 70 chunks of 256
+    # the larger of the K-mean partials (70 chunks of 256) and the V statistics + residual sums (18 chunks of 1024, 278 tiles)
+    assert lib.paro_prep_workspace_bytes(2, 48, 17776, 64) == 2 * 48 * (18 * 3 + 278 * 2) * 64 * 4
 
     def prep(D=64, N=128, grid=(2, 8, 8), n_text=0, q=p, ws=p, ws_bytes=1 << 20):
         return lib.paro_rope_permute_quant_fwd(q, p, p, 0, None, None, p, None, p, p, p, p, p, p, p, ws, ws_bytes,

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import cosine
+from conftest import cosine, untile_v8, v8_offset_expected
 from oracle import paro_oracle as O
 
 FIX = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "path_small.npz")
@@ -107,19 +107,14 @@ def test_hip_path_matches_the_fixture(fx, dev):
     # mean's last bit moves a value across a rounding boundary
     v8, vsc, vm = Q.per_channel_fp8(vp)
     assert np.array_equal(vsc.cpu().numpy(), fx["v_scale"])
-    assert np.allclose(vm.cpu().numpy(), fx["v_mean"], atol=1e-7, rtol=1e-5)
-    tiles = v8.view(torch.uint8).flatten().cpu().numpy().reshape(B, H, -1, D // 32, 2, 64, 16)
-    nbk = tiles.shape[2]
-    tok = np.zeros((B, H, nbk * 64, D), dtype=np.uint8)
-    for dt in range(D // 32):
-        for mt in range(2):
-            for lane in range(64):
-                for r in range(16):
-                    t = 32 * mt + 8 * (r // 4) + 4 * (lane // 32) + r % 4
-                    tok[:, :, t::64, 32 * dt + lane % 32][:, :, :nbk] = tiles[:, :, :, dt, mt, lane, r]
+    tok = untile_v8(v8, B, H, N, D)
     assert (tok[:, :, N:] == 0).all()
-    diff = np.abs(tok[:, :, :N].astype(np.int32) - fx["v8"].astype(np.int32))
+    diff = np.abs(tok[:, :, :N].numpy().astype(np.int32) - fx["v8"].astype(np.int32))
     assert diff.max() <= 1 and (diff != 0).mean() <= 1e-3
+    # the offset the epilogue adds back: the fixture's mean plus the mean rounding residual of these codes
+    want = v8_offset_expected(_f16(fx["v_perm"]), tok, vsc)
+    assert np.allclose(vm.cpu().double().numpy(), want.numpy(), atol=1e-5, rtol=1e-5)
+    assert (np.abs(vm.cpu().numpy() - fx["v_mean"]) <= 1e-6 + 16.0 * fx["v_scale"]).all()
     # integer scores through the debug dump of the attention kernel
     mask = torch.from_numpy(fx["mask"]).to(dev)
     nb = (N + 63) // 64

@@ -189,3 +189,70 @@ def test_nhd_layout_and_paroattn_entry(dev):
     # against attention on the UNQUANTISED tensors: INT8 Q/K (K smoothed) and FP8 P/V together
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
     assert cosine(dense.cpu(), ref) >= 0.998
+
+
+def _ramp_case(B, H, N, D, dtype, seed, pattern):
+    """Scores that climb along the key axis, so that later kept blocks exceed the running row maximum by
+    more than the FP8 headroom (3.75 octaves) again and again: "ramp" adds a common direction w to every
+    query and b*w*step to the keys of block b (each block ~4.3 octaves above the one before); "spike" puts
+    single keys 12 and 25 octaves above the rest into late blocks."""
+    q, k, v = synth.make_qkv(B, H, N, D, dtype, seed=seed, k_bias_std=0.0)
+    g = torch.Generator().manual_seed(seed + 100)
+    w = torch.randn(D, generator=g)
+    w = w / w.norm()
+    qf, kf = q.float() * 0.3 + 4.0 * w, k.float() * 0.3
+    blk = torch.arange(N) // 64
+    sm = D ** -0.5
+    if pattern == "ramp":
+        kf = kf + (3.0 * blk.float() / (4.0 * sm))[None, None, :, None] * w     # +3 nats per block
+    else:
+        for j, nats in ((N // 2 + 5, 8.0), (N - 70, 17.0)):
+            kf[:, :, j] += (nats / (4.0 * sm)) * w
+    return qf.to(dtype), kf.to(dtype), v
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("pattern,causal,density", [("ramp", False, 1.0), ("ramp", False, 0.5), ("ramp", True, 1.0),
+                                                    ("spike", False, 0.5), ("spike", True, 1.0)])
+def test_fast_path_maximum_recovery(dev, D, pattern, causal, density):
+    """The default (fast) softmax path computes a block's weights against the running maximum as it is
+    and only afterwards notices, from the largest 16-bit field it built, that a score was more than the
+    FP8 headroom above it; it then refreshes the maximum and recomputes the block.  Here that happens in
+    block after block (every row, dense, sparse and causal masks): the output must be finite and match
+    both the oracle and the exact-exponential path."""
+    import paroatten_amd as P
+    B, H, N = 1, 2, 1024 - 19
+    nb = (N + 63) // 64
+    q, k, v = _ramp_case(B, H, N, D, torch.float16, 7 + D, pattern)
+    mask = (torch.ones(H, nb, nb, dtype=torch.bool) if density == 1.0
+            else synth.make_block_mask(H, nb, density, seed=5))
+    q8, qs, k8, ks = O.per_warp_int8(q, k, BLKQ=64, WARPQ=32, BLKK=64)
+    o_ref, _ = O.sparse_attention(q8, k8, v, qs, ks, mask[None], D ** -0.5, is_causal=causal, out_dtype=torch.float32)
+    # rows that one or a few keys dominate: the error is FP8's relative rounding error on each product
+    # p*v (at most 2^-4 for V's code and for P's), so the elementwise bound is 0.125 * sum_j p_ij |v_j|
+    a_ref, _ = O.sparse_attention(q8, k8, v.abs(), qs, ks, mask[None], D ** -0.5, is_causal=causal,
+                                  out_dtype=torch.float32)
+
+    def close(a, b):
+        e = (a.float() - b.float()).abs()
+        assert bool((e <= ATOL + 0.125 * a_ref).all()), float((e - 0.125 * a_ref).max())
+        assert cosine(a, b) >= COS, cosine(a, b)
+    # the case does what it is meant to: block maxima climb by more than the headroom many times per row
+    s = O.qk_int32(q8, k8)[0, 0].double() * qs[0, 0].double().repeat_interleave(32)[:N, None] \
+        * ks[0, 0].double().repeat_interleave(64)[None, :N] * (D ** -0.5) * O.LOG2E
+    keep = O.expand_block_mask(mask[0], N, N)
+    if causal:
+        keep = keep & (torch.arange(N)[None, :] <= torch.arange(N)[:, None])
+    s = s.masked_fill(~keep, float("-inf"))
+    pad = torch.full((N, nb * 64 - N), float("-inf"), dtype=s.dtype)
+    blockmax = torch.cat([s, pad], dim=1).reshape(N, nb, 64).amax(dim=-1)
+    run = torch.cummax(blockmax, dim=1).values
+    jumps = ((blockmax[:, 1:] - run[:, :-1]) > 3.75).sum(dim=1)
+    assert int(jumps.max()) >= (1 if pattern == "spike" else 4), int(jumps.max())
+    kw = dict(is_causal=causal, smooth_k=False)
+    o_fast = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), **kw).cpu()
+    o_exact = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), exact_exp=True, **kw).cpu()
+    assert torch.isfinite(o_fast.float()).all() and torch.isfinite(o_exact.float()).all()
+    close(o_fast, o_ref)
+    close(o_exact, o_ref)
+    close(o_fast, o_exact)

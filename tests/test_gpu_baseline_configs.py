@@ -35,8 +35,12 @@ def _check_heads(dev, wl, density, heads, seed, n_heads_total=None, with_rope=Fa
     from paroatten_amd import rope
     H = n_heads_total or len(heads)
     B, N, D, nb = 1, wl.N, wl.D, wl.nb
-    q, k, v = synth.make_qkv(B, H, N, D, wl.dtype, seed=seed)
-    mask = synth.make_block_mask(H, nb, density, seed=seed + 1)
+    if H > 8:   # a full extent: generated on the device, the heads to check copied back
+        q, k, v = (t.cpu() for t in synth.make_qkv_device(B, H, N, D, wl.dtype, seed=seed, device=dev))
+        mask = synth.make_block_mask(H, nb, density, seed=seed + 1, device=dev).cpu()
+    else:
+        q, k, v = synth.make_qkv(B, H, N, D, wl.dtype, seed=seed)
+        mask = synth.make_block_mask(H, nb, density, seed=seed + 1)
     plan = synth.make_permute_plan(1, H, seed=seed + 2)
     cos = sin = None
     if with_rope:
@@ -71,9 +75,17 @@ def test_cfg2_whole_path_with_rope(dev):
     _check_heads(dev, synth.WORKLOADS["cogvideox5b"], 0.3, heads=[1], seed=77, n_heads_total=2, with_rope=True)
 
 
-def test_cfg3_wan480p_head(dev):
-    """config 3: D=128, bf16, N=32760 (21x30x52), density 0.3."""
-    _check_heads(dev, synth.WORKLOADS["wan14b_480p"], 0.3, heads=[1], seed=33, n_heads_total=2)
+def test_cfg3_wan480p_full_extent(dev):
+    """config 3 at its full extent: B=1, H=40, D=128, bf16, N=32760 (21x30x52), density 0.3; two of
+    the 40 heads checked in full against the oracle."""
+    wl = synth.WORKLOADS["wan14b_480p"]
+    _check_heads(dev, wl, 0.3, heads=[7, 39], seed=33, n_heads_total=wl.H)
+
+
+def test_cfg0_whole_path_with_permutation(dev):
+    """config 0 as the benchmark list states it: B=1, H=2, D=64, fp16, a 16x16x16 grid (N=4096), K bias,
+    density 0.5, a random F/H/W order per head applied before the attention and inverted after."""
+    _check_heads(dev, synth.WORKLOADS["cfg0_plumbing"], 0.5, heads=[0, 1], seed=0)
 
 
 def test_cfg1_rope_permute_full_shape(dev):
@@ -135,51 +147,50 @@ def test_cfg2_full_extent_properties(dev):
     assert cosine(o[0, 7].cpu(), ref.cpu()) >= COS
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-def test_cfg4_wan720p_rows(dev, dtype):
-    """config 4: D=128, N=75600 (21x45x80), density 0.2 and the dense mask: one head on the GPU at full
-    length; the oracle checks three whole q-blocks of it (rows are independent).
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_cfg4_wan720p_full_extent(dev, dtype):
+    """config 4 at its full extent: B=1, H=40, D=128, N=75600 (21x45x80), density 0.2 and the dense mask,
+    in the configuration's own dtype (bfloat16) and in float16.  All 40 heads run; for three of them
+    the oracle checks three whole q-blocks (rows are independent): atol 2e-2 and cosine >= 0.999.
 
-    With i.i.d. V the output of a row that averages n tokens is a random walk of size ~|v|/sqrt(n_eff):
-    5e-3..1e-2 here, far below atol, so the relative measures are the ones that bite.
-      * float16 V: the FP8 budget (2.65% for V, 2.65..3.1% for P) is independent of n: cosine >= 0.999.
-      * bfloat16 V (config 4's dtype): v - mean(v) of an 8-bit-significand lattice is not symmetric
-        about the e4m3 cells, so the quantised channel keeps a mean error of ~2.7e-4 |v| that does not
-        shrink with n (3x the 1/sqrt(n) value at n = 75600; measured on the oracle's per_channel_fp8,
-        same for any implementation of mean-smoothed e4m3 V).  Against a signal of 6e-3 that alone is
-        4.5%, so the bound is stated as rms error <= 4.5% of the signal + 4e-4 of rms(v)."""
+    With i.i.d. V the output of a row that averages n keys is of size |v|/sqrt(n_eff), 5e-3..1e-2 here,
+    far below atol, so the cosine is the measure that bites: it holds because the per-channel mean
+    rounding residual of the FP8 codes (which does not shrink with n, and which the 8-significant-bit
+    lattice of bfloat16 makes ~3e-4 |v|) is folded into the offset the epilogue adds back."""
     from paroatten_amd import _qattn_sm80 as qattn
     from paroatten_amd import permute as PM
     from paroatten_amd import quant as Q
     wl = synth.WORKLOADS["wan14b_720p"]
-    N, D, nb = wl.N, wl.D, wl.nb
-    q, k, v = synth.make_qkv(1, 1, N, D, dtype, seed=44)
-    plan = synth.make_permute_plan(1, 1, seed=45)
+    H, N, D, nb = wl.H, wl.N, wl.D, wl.nb
+    q, k, v = synth.make_qkv_device(1, H, N, D, dtype, seed=44, device=dev)
+    plan = synth.make_permute_plan(1, H, seed=45)
     orders = PM.head_orders(plan, 0, dev)
-    qp, kp, vp = PM.rope_permute(q.to(dev), k.to(dev), v.to(dev), orders, wl.grid, 0)
-    rq, rk, rv = O.permute_qk(q, k, v, plan, 0, wl.grid, 0)
-    assert torch.equal(qp.cpu(), rq) and torch.equal(vp.cpu(), rv)
-    km = rk.float().mean(dim=2, keepdim=True).to(rk.dtype)
-    q8, qs, k8, ks = O.per_warp_int8(rq, rk, km=km, BLKQ=64, WARPQ=32, BLKK=64)
-    # same K mean on both sides (a one-ulp difference of a 16-bit mean would give two different,
-    # equally valid int8 quantisations, whose difference is not what this test measures)
-    g8 = Q.per_warp_int8(qp, kp, km.to(dev), BLKQ=64, WARPQ=32, BLKK=64)
-    assert torch.equal(g8[0].cpu(), q8) and torch.equal(g8[2].cpu(), k8)
-    blocks = [0, 500, 1180]
+    qp, kp, vp = PM.rope_permute(q, k, v, orders, wl.grid, 0)
+    del q, k, v
+    # the same rounded K mean on both sides (a one-ulp difference of a 16-bit mean would give two
+    # different, equally valid int8 quantisations, whose difference is not what this test measures)
+    km = kp.float().mean(dim=2, keepdim=True).to(dtype)
+    g8 = Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64)
+    heads, blocks = [0, 17, 39], [0, 500, 1180]
     rows = torch.cat([torch.arange(64 * b, 64 * b + 64) for b in blocks])
-    qs_sel = torch.cat([qs[:, :, 2 * b:2 * b + 2] for b in blocks], dim=-1)
-    v_rms = rv.float().pow(2).mean().sqrt().item()
+    refs = {}
+    for h in heads:
+        rq, rk, rv = qp[:, h:h + 1].cpu(), kp[:, h:h + 1].cpu(), vp[:, h:h + 1].cpu()
+        q8, qs, k8, ks = O.per_warp_int8(rq, rk, km=km[:, h:h + 1].cpu(), BLKQ=64, WARPQ=32, BLKK=64)
+        assert torch.equal(g8[0][:, h:h + 1].cpu(), q8) and torch.equal(g8[2][:, h:h + 1].cpu(), k8)
+        assert torch.equal(g8[1][:, h:h + 1].cpu(), qs) and torch.equal(g8[3][:, h:h + 1].cpu(), ks)
+        refs[h] = (q8[:, :, rows], k8, rv, torch.cat([qs[:, :, 2 * b:2 * b + 2] for b in blocks], dim=-1), ks)
     for density in (0.2, 1.0):
-        mask = synth.make_block_mask(1, nb, density, seed=46) if density < 1 else torch.ones(1, nb, nb, dtype=torch.bool)
+        mask = (synth.make_block_mask(H, nb, density, seed=46, device=dev) if density < 1
+                else torch.ones(H, nb, nb, dtype=torch.bool, device=dev))
         o = torch.empty_like(qp)
-        qattn.qk_int8_sv_f16_accum_f16_attn(g8[0], g8[2], vp, o, g8[1], g8[3], 1, 0, 2, D ** -0.5, 0, mask.to(dev))
-        o = o.cpu()
-        ref, _ = O.sparse_attention(q8[:, :, rows], k8, rv, qs_sel, ks, mask[None][:, :, blocks], D ** -0.5,
-                                    out_dtype=torch.float32)
-        got = o[:, :, rows].float()
-        assert (got - ref).abs().max().item() <= ATOL
-        err_rms = (got - ref).pow(2).mean().sqrt().item()
-        ref_rms = ref.pow(2).mean().sqrt().item()
-        if dtype == torch.float16:
-            assert cosine(got, ref) >= COS, (density, cosine(got, ref))
-        assert err_rms <= 0.045 * ref_rms + 4e-4 * v_rms, (density, err_rms, ref_rms)
+        qattn.qk_int8_sv_f16_accum_f16_attn(g8[0], g8[2], vp, o, g8[1], g8[3], 1, 0, 2, D ** -0.5, 0, mask)
+        assert torch.isfinite(o.float()).all()
+        for h in heads:
+            q8r, k8, rv, qs_sel, ks = refs[h]
+            ref, _ = O.sparse_attention(q8r, k8, rv, qs_sel, ks, mask[None, h:h + 1][:, :, blocks].cpu(), D ** -0.5,
+                                        out_dtype=torch.float32)
+            got = o[:, h:h + 1][:, :, rows].cpu().float()
+            err = (got - ref).abs().max().item()
+            assert err <= ATOL, (density, h, err)
+            assert cosine(got, ref) >= COS, (density, h, cosine(got, ref))
