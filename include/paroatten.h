@@ -233,6 +233,22 @@ int paro_rope_k_mean(const void* k, int dtype, const float* cos, const float* si
                      int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
                      int64_t mean_stride_b, int64_t mean_stride_h, void* stream);
 
+/* paro_rope_k_mean for callers that can neither allocate device memory nor bring a workspace (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments and results as paro_rope_k_mean without the workspace: the per-chunk partial
+ * sums go to a work buffer built into the library (a __device__ array of
+ * PARO_ROPE_K_MEAN_STATIC_MAX_FLOATS floats = 8 MiB that every GPU the library runs on holds until the
+ * process ends).  The call allocates and frees nothing.  B * H * ceil(N/256) * D must not exceed
+ * PARO_ROPE_K_MEAN_STATIC_MAX_FLOATS (PARO_ERR_RUNTIME otherwise; CogVideoX-5b needs 0.43 M, Wan 720p
+ * 1.5 M).  All calls on one GPU share that GPU's buffer: calls that may overlap on one GPU (different
+ * streams, different threads) race; calls on one stream do not.  The first call on each device looks the
+ * buffer's address up (hipGetSymbolAddress) and should therefore be made outside stream capture. */
+#define PARO_ROPE_K_MEAN_STATIC_MAX_FLOATS (2 * 1024 * 1024)
+int paro_rope_k_mean_static(const void* k, int dtype, const float* cos, const float* sin, void* k_mean,
+                            int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                            int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                            int64_t mean_stride_b, int64_t mean_stride_h, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * V helpers kept for API completeness of paroattention._fused (csrc/fused/fused.cu:200-260,
  * 770-848): out_f16[b,h,n,:] = fp16(v - mean[b,h,:]) (bf16 input: subtract in bf16 first).

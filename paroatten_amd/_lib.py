@@ -59,6 +59,8 @@ SIGNATURES = {
                                             _L, _L, _I, _P]),
     "paro_rope_k_mean": (c_int, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _I,
                                  _L, _L, _L, _L, _L, _P]),
+    "paro_rope_k_mean_static": (c_int, [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,
+                                        _L, _L, _L, _L, _L, _P]),
     "paro_mask_bits_bytes": (c_int64, [_L]),
     "paro_mask_pack": (c_int, [_P, _P, _L, _P]),
     "paro_mask_unpack": (c_int, [_P, _P, _L, _P]),

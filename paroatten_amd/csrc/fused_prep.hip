@@ -19,8 +19,35 @@
 // (paroattention/cogvideox.py:167-186), QuantInt8Kernel (csrc/fused/fused.cu:64-198) and
 // MeanScaleKernel (csrc/fused/fused.cu:316-427).
 #include "paro_device.hpp"
+#include <mutex>
 
 namespace paro {
+
+// Library-owned work buffer of paro_rope_k_mean_static (the per-chunk partial sums of the K mean), for
+// callers that can neither allocate nor bring a workspace.  One copy per GPU, at its own address, held
+// from the moment the code object is loaded on that GPU until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; the address kernels get is looked up once per
+// device (with that device current) and kept in g_kmean_scratch.
+constexpr int64_t KMEAN_SCRATCH_FLOATS = PARO_ROPE_K_MEAN_STATIC_MAX_FLOATS;   // 8 MiB
+static __device__ __align__(256) float scratch[KMEAN_SCRATCH_FLOATS];
+constexpr int MAX_DEVICES = 64;
+static float* g_kmean_scratch[MAX_DEVICES];
+static std::mutex g_kmean_scratch_mu;
+
+static int kmean_scratch_of_current_device(float** out) {
+  int dev = -1;
+  PARO_HIP(hipGetDevice(&dev));
+  PARO_CHECK(dev >= 0 && dev < MAX_DEVICES, PARO_ERR_RUNTIME, "paro_rope_k_mean_static: device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_kmean_scratch_mu);
+  if (g_kmean_scratch[dev] == nullptr) {
+    void* ptr = nullptr;
+    PARO_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    PARO_CHECK(ptr != nullptr, PARO_ERR_HIP, "paro_rope_k_mean_static: no device address for the scratch array");
+    g_kmean_scratch[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_kmean_scratch[dev];
+  return PARO_OK;
+}
 
 // LDS of the preparation kernel.  The gathered token rows never pass through registers on their way
 // in: LDS-DMA buffer loads drop them into a ring of four 64-token tile slots, Q, K, V of one (batch,
@@ -478,6 +505,26 @@ extern "C" int paro_rope_k_mean(const void* k, int dtype, const float* cos, cons
 #undef PARO_KM
   PARO_HIP(hipGetLastError());
   return PARO_OK;
+}
+
+extern "C" int paro_rope_k_mean_static(const void* k, int dtype, const float* cos, const float* sin, void* k_mean,
+                                       int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                                       int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                       int64_t mean_stride_b, int64_t mean_stride_h, void* stream) {
+  using namespace paro;
+  PARO_CHECK(B > 0 && H > 0 && N > 0 && (D == 64 || D == 128), PARO_ERR_INVALID_VALUE,
+             "Unsupported shape or head dim: B=%d H=%d N=%d D=%d", B, H, N, D);
+  const int64_t need = (int64_t)B * H * ceil_div(N, K_CHUNK) * D;
+  PARO_CHECK(need <= KMEAN_SCRATCH_FLOATS, PARO_ERR_RUNTIME,
+             "paro_rope_k_mean_static: B*H*ceil(N/%d)*D = %lld partial sums exceed the built-in work buffer of %lld "
+             "floats; use paro_rope_k_mean with a workspace of its own",
+             K_CHUNK, (long long)need, (long long)KMEAN_SCRATCH_FLOATS);
+  float* ws = nullptr;
+  if (int rc = kmean_scratch_of_current_device(&ws)) return rc;
+  // every partial sum the second launch reads is written by the first: nothing of the buffer has to
+  // start at zero, whatever the previous call left in it
+  return paro_rope_k_mean(k, dtype, cos, sin, k_mean, ws, KMEAN_SCRATCH_FLOATS * 4, B, H, N, D, n_text, F, Hh, W,
+                          k_stride_b, k_stride_h, k_stride_n, mean_stride_b, mean_stride_h, stream);
 }
 
 extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const void* v, int dtype, const float* cos,
