@@ -260,6 +260,33 @@ int paro_sub_mean(const void* v, int dtype, const void* mean, void* out_f16,
                   int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * V preparation in the reference's own storage format, for callers of paroattention._fused.
+ * paro_transpose_pad_permute stands in for transpose_pad_permute_cuda (csrc/fused/fused.cu:262-313,
+ * 850-923): in [B,H,N,D] 16-bit through (stride_b, stride_h, stride_n) -> out [B,H,D,ceil64(N)] through
+ * (stride_b, stride_h, stride_d), last dim contiguous; tokens >= N are zero; inside every group of 16
+ * tokens, position i holds token [0,1,8,9,2,3,10,11,4,5,12,13,6,7,14,15][i] (the operand order of NVIDIA's
+ * fp8 mma, paroattention/quant.py:231-234; this library's attention kernel reads paro_v_fp8_pack's tiles
+ * instead).  D in {64,128}.
+ * paro_channel_quant_fp8 stands in for scale_fuse_quant_cuda (mean == NULL) and mean_scale_fuse_quant_cuda
+ * (fused.cu:316-427, 925-1083): per row in[b,h,d,:] of row_len entries,
+ *   n16 = ceil16(num_tokens); mean = sum(in[:n16]) / n16 (0 without `mean`)
+ *   amax = max(|max(in[:n16]) - mean|, |min(in[:n16]) - mean|) ; scale = amax / scale_max
+ *   out[:ceil64(num_tokens)] = e4m3_rne_satfinite((in - mean) * (scale_max / amax))
+ * as the reference does it (the zero padding up to n16 takes part in the statistics).  A constant row
+ * gives zero codes (the reference divides by zero there).  mean, scale: fp32 [B,H,D] through (stride_b,
+ * stride_h).
+ * ------------------------------------------------------------------------------------------- */
+int paro_transpose_pad_permute(const void* in, void* out, int dtype, int B, int H, int N, int D,
+                               int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_n,
+                               int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_d, void* stream);
+int paro_channel_quant_fp8(const void* in, int dtype, uint8_t* out, float* mean, float* scale,
+                           int B, int H, int D, int num_tokens, int row_len, float scale_max,
+                           int64_t in_stride_b, int64_t in_stride_h, int64_t in_stride_d,
+                           int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_d,
+                           int64_t mean_stride_b, int64_t mean_stride_h,
+                           int64_t scale_stride_b, int64_t scale_stride_h, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * Block-mask bit packing.  The sparse plan is the one operand of the path that is staged from the
  * host per layer (paroattention/prefetch_utils.py:34-59 keeps it as torch.bool on the CPU and
  * paroattention/cogvideox.py:188-213 copies one [H,nb,nb] slice per call); as bits it is 8x smaller

@@ -22,6 +22,11 @@ Pinning status
         itself is pinned; the TABLE CONSTRUCTION is "parity unpinned" (third-party diffusers,
         no version pinned by the reference, not importable here)
   per_channel_fp8                             : pinned against torch.float8_e4m3fn casting
+  transpose_pad_permute                       : pinned (torch.transpose + pad library routines; the
+        within-16 order is stated twice by the reference, as a formula in the kernel and as a
+        literal list in a docstring, and the two are checked against each other)
+  channel_quant_fp8                           : pinned (float64 statistics, torch.float8_e4m3fn
+        casting; reduces to per_channel_fp8 when the token count is a multiple of 16)
 """
 from __future__ import annotations
 
@@ -339,9 +344,52 @@ def per_channel_fp8(v: torch.Tensor, scale_max: float = 448.0, smooth_v: bool = 
     amax = vf.abs().amax(dim=2)
     scale = amax / scale_max
     # fused.cu:399,414: multiply by recp_scale = scale_max / amax (a constant channel gives 0, not NaN)
-    recp = torch.where(amax > 0, scale_max / amax, torch.zeros_like(amax))
+    # a tensor / tensor quotient: a Python scalar divided by a tensor is evaluated as reciprocal-times-
+    # scalar, which rounds twice
+    recp = torch.where(amax > 0, torch.full_like(amax, scale_max) / amax, torch.zeros_like(amax))
     v8 = (vf * recp.unsqueeze(2)).clamp(-scale_max, scale_max).to(torch.float8_e4m3fn)
     return v8, scale, vm
+
+
+# paroattention/quant.py:231-234 (docstring of per_channel_fp8): position i of every group of 16
+# tokens holds token V_SHUFFLE16[i]
+V_SHUFFLE16 = (0, 1, 8, 9, 2, 3, 10, 11, 4, 5, 12, 13, 6, 7, 14, 15)
+
+
+def shuffle16_position_of(r: int) -> int:
+    """where TransposePadPermuteKernel puts token r of a group of 16 (csrc/fused/fused.cu:287-291:
+    smem_load_row = (r / 8) * 2 + ((r / 2) % 4) * 4 + r % 2)."""
+    return (r // 8) * 2 + ((r // 2) % 4) * 4 + r % 2
+
+
+def transpose_pad_permute(v: torch.Tensor) -> torch.Tensor:
+    """transpose_pad_permute_cuda for the HND layout (csrc/fused/fused.cu:262-313, 850-923):
+    [B,H,N,D] -> [B,H,D,ceil64(N)], zero padding, tokens inside every group of 16 reordered."""
+    B, H, N, D = v.shape
+    padded = (N + 63) // 64 * 64
+    x = torch.nn.functional.pad(v.transpose(2, 3), (0, padded - N))          # [B,H,D,padded]
+    src = torch.arange(padded).view(-1, 16)[:, list(V_SHUFFLE16)].reshape(-1)   # out[i] = in[src[i]]
+    return x[..., src].contiguous()
+
+
+def channel_quant_fp8(x: torch.Tensor, num_tokens: int, scale_max: float = 448.0, sub_mean: bool = True):
+    """MeanScaleKernel behind mean_scale_fuse_quant_cuda / scale_fuse_quant_cuda
+    (csrc/fused/fused.cu:316-427): x [B,H,D,L] 16-bit rows.  Statistics over the first
+    n16 = ceil16(num_tokens) entries (:335-336: the zero padding takes part, and the mean divides by
+    n16, :381); amax = max(|max - mean|, |min - mean|) (:385); scale = amax / scale_max (:393);
+    codes for the first ceil64(num_tokens) entries: e4m3((x - mean) * (scale_max / amax)) (:399-421).
+    Returns (codes float8 [B,H,D,ceil64], scale f32 [B,H,D], mean f32 [B,H,D] or None).  A constant row
+    gives zero codes (the reference divides by zero there)."""
+    n16 = (num_tokens + 15) // 16 * 16
+    n64 = (num_tokens + 63) // 64 * 64
+    xf = x.to(torch.float32)
+    head = xf[..., :n16]
+    mean = (head.double().sum(dim=-1) / n16).float() if sub_mean else torch.zeros(x.shape[:-1])
+    amax = torch.maximum((head.amax(dim=-1) - mean).abs(), (head.amin(dim=-1) - mean).abs())
+    scale = amax / scale_max
+    recp = torch.where(amax > 0, torch.full_like(amax, scale_max) / amax, torch.zeros_like(amax))   # one rounding
+    codes = ((xf[..., :n64] - mean.unsqueeze(-1)) * recp.unsqueeze(-1)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return codes, scale, (mean if sub_mean else None)
 
 
 # ----------------------------------------------------------------------------------------

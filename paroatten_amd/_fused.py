@@ -132,20 +132,81 @@ def sub_mean_cuda(input, mean, output, tensor_layout):
                                output.stride(0), os_h, os_n, stream_of(input))
 
 
-_NV_LAYOUT = (
-    "{name} writes V in the register-fragment order of NVIDIA's fp8 mma "
-    "(csrc/fused/fused.cu:287-291); that order has no meaning on gfx950 and nothing consumes it. "
-    "Use paroatten_amd.quant.per_channel_fp8, which produces FP8 V in this library's MFMA tile order."
-)
-
-
 def transpose_pad_permute_cuda(input, output, tensor_layout):
-    raise NotImplementedError(_NV_LAYOUT.format(name="transpose_pad_permute_cuda"))
+    """csrc/fused/fused.cu:850-923: input [B,H,N,D] (layout 1) or [B,N,H,D] (layout 0) ->
+    output [B,H,D,ceil64(N)] or [B,D,H,ceil64(N)], tokens >= N zero, tokens inside every group of 16
+    in the order 0,1,8,9,2,3,10,11,4,5,12,13,6,7,14,15 (the operand order of NVIDIA's fp8 mma; this
+    library's attention kernel reads the tiles of quant.per_channel_fp8 instead)."""
+    _check_cuda(input, "input")
+    _check_cuda(output, "output")
+    _chk(input.stride(-1) == 1, "Tensor input must be contiguous at the last dimension")
+    _chk(output.is_contiguous(), "Tensor output must be contiguous")
+    _chk(input.dim() == 4, "Tensor input must have dimension number (4)")
+    _chk(output.dim() == 4, "Tensor output must have dimension number (4)")
+    B, D = input.size(0), input.size(3)
+    N, H, is_n, is_h = _layout_dims(input, tensor_layout)
+    padded = (N + 63) // 64 * 64
+    if tensor_layout == 0:
+        _chk(tuple(output.shape) == (B, D, H, padded),
+             "Tensor output must have shape (batch_size, head_dim, num_heads, padded_num_tokens)")
+        os_d, os_h = output.stride(1), output.stride(2)
+    else:
+        _chk(tuple(output.shape) == (B, H, D, padded),
+             "Tensor output must have shape (batch_size, num_heads, head_dim, padded_num_tokens)")
+        os_d, os_h = output.stride(2), output.stride(1)
+    _chk(input.dtype == output.dtype, "Input and output must have the same data type")
+    if input.dtype not in _HALF:
+        raise RuntimeError(f"transpose_pad_permute_cuda failed to dispatch data type {input.dtype}")
+    if D not in (64, 128):
+        raise ValueError(f"Unsupported head dim: {D}")
+    _lib.on(input).paro_transpose_pad_permute(ptr(input), ptr(output), _lib.DTYPE_CODE[input.dtype], B, H, N, D,
+                                            input.stride(0), is_h, is_n, output.stride(0), os_h, os_d,
+                                            stream_of(input))
+
+
+def _channel_quant(input, output, mean, scale, num_tokens, scale_max, tensor_layout, fn_name):
+    tensors = [(input, "input"), (output, "output")] + ([(mean, "mean")] if mean is not None else []) + [(scale, "scale")]
+    for t, n in tensors:
+        _check_cuda(t, n)
+    if mean is not None:
+        _chk(mean.dtype == torch.float32, "Tensor mean must have dtype (torch::kFloat)")
+    _chk(scale.dtype == torch.float32, "Tensor scale must have dtype (torch::kFloat)")
+    for t, n in tensors:
+        _chk(t.is_contiguous(), f"Tensor {n} must be contiguous")
+    _chk(input.dim() == 4, "Tensor input must have dimension number (4)")
+    _chk(output.dim() == 4, "Tensor output must have dimension number (4)")
+    if mean is not None:
+        _chk(mean.dim() == 3, "Tensor mean must have dimension number (3)")
+    _chk(scale.dim() == 3, "Tensor scale must have dimension number (3)")
+    B, row_len = input.size(0), input.size(3)
+    if tensor_layout == 0:
+        H, D, d_dim, h_dim = input.size(2), input.size(1), 1, 2
+    else:
+        H, D, d_dim, h_dim = input.size(1), input.size(2), 2, 1
+    _chk(tuple(output.shape) == tuple(input.shape),
+         "Tensor output must have shape (input.size(0), input.size(1), input.size(2), input.size(3))")
+    if mean is not None:
+        _chk(tuple(mean.shape) == (B, H, D), "Tensor mean must have shape (batch_size, num_heads, head_dim)")
+    _chk(tuple(scale.shape) == (B, H, D), "Tensor scale must have shape (batch_size, num_heads, head_dim)")
+    if input.dtype not in _HALF:
+        raise RuntimeError(f"{fn_name} failed to dispatch data type {input.dtype}")
+    # the reference leaves the output dtype unchecked (a commented-out int8 check): one byte per entry
+    _chk(output.element_size() == 1, "Tensor output must have a one-byte dtype (torch.float8_e4m3fn)")
+    ms_b, ms_h = (mean.stride(0), mean.stride(1)) if mean is not None else (0, 0)
+    _lib.on(input).paro_channel_quant_fp8(
+        ptr(input), _lib.DTYPE_CODE[input.dtype], ptr(output), ptr(mean), ptr(scale), B, H, D, int(num_tokens), row_len,
+        float(scale_max), input.stride(0), input.stride(h_dim), input.stride(d_dim),
+        output.stride(0), output.stride(h_dim), output.stride(d_dim), ms_b, ms_h,
+        scale.stride(0), scale.stride(1), stream_of(input))
 
 
 def scale_fuse_quant_cuda(input, output, scale, num_tokens, scale_max, tensor_layout):
-    raise NotImplementedError(_NV_LAYOUT.format(name="scale_fuse_quant_cuda"))
+    """csrc/fused/fused.cu:925-1000: per (batch, head, channel) row of the transposed V:
+    scale = max|x[:ceil16(num_tokens)]| / scale_max, output = e4m3(x * scale_max / max|x|)."""
+    _channel_quant(input, output, None, scale, num_tokens, scale_max, tensor_layout, "scale_fuse_quant_cuda")
 
 
 def mean_scale_fuse_quant_cuda(input, output, mean, scale, num_tokens, scale_max, tensor_layout):
-    raise NotImplementedError(_NV_LAYOUT.format(name="mean_scale_fuse_quant_cuda"))
+    """csrc/fused/fused.cu:1002-1083: as scale_fuse_quant_cuda after subtracting the row mean
+    (sum over the first ceil16(num_tokens) entries divided by that count, fused.cu:335,381)."""
+    _channel_quant(input, output, mean, scale, num_tokens, scale_max, tensor_layout, "mean_scale_fuse_quant_cuda")

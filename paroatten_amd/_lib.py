@@ -64,6 +64,9 @@ SIGNATURES = {
     "paro_mask_bits_bytes": (c_int64, [_L]),
     "paro_mask_pack": (c_int, [_P, _P, _L, _P]),
     "paro_mask_unpack": (c_int, [_P, _P, _L, _P]),
+    "paro_transpose_pad_permute": (c_int, [_P, _P, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
+    "paro_channel_quant_fp8": (c_int, [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F,
+                                       _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
     "paro_sub_mean": (c_int, [_P, _I, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
 }
 

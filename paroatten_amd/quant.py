@@ -76,7 +76,8 @@ def sub_mean(v: torch.Tensor, tensor_layout: str = "HND"):
     return v_smoothed, vm
 
 
-def per_channel_fp8(v: torch.Tensor, tensor_layout: str = "HND", scale_max: float = 448.0, smooth_v: bool = True):
+def per_channel_fp8(v: torch.Tensor, tensor_layout: str = "HND", scale_max: float = 448.0, smooth_v: bool = True,
+                    tile_order: bool = True):
     """V -> float8_e4m3fn with one scale (and, if smooth_v, one mean) per (batch, head, channel)
     (paroattention/quant.py:224-293).  Returns (v_fp8, v_scale [B,H,D] f32, vm [B,H,D] f32 or None).
 
@@ -84,7 +85,27 @@ def per_channel_fp8(v: torch.Tensor, tensor_layout: str = "HND", scale_max: floa
     byte count, but its bytes are in the 64-token MFMA tile order this library's attention kernel
     reads (include/paroatten.h, paro_v_fp8_pack), grouped [B,H,tile,...] for either layout, where
     the reference's are in the fragment order of NVIDIA's fp8 mma.  The mean divides by the true
-    token count."""
+    token count, and `vm` is the offset the attention epilogue adds back: that mean plus the mean rounding
+    residual of the channel's codes.
+
+    tile_order=False runs the reference's own sequence instead (transpose_pad_permute_cuda, then
+    mean_scale_fuse_quant_cuda or scale_fuse_quant_cuda): bytes in the reference's order, statistics over
+    ceil16(N) tokens, any scale_max.  Nothing in this library consumes that form."""
+    if not tile_order:
+        b, h, n, d = _dims(v, tensor_layout)
+        layout_flag = 0 if tensor_layout == "NHD" else 1
+        padded = (n + 63) // 64 * 64
+        shape = (b, h, d, padded) if tensor_layout == "HND" else (b, d, h, padded)
+        vt = torch.empty(shape, dtype=v.dtype, device=v.device)
+        _fused.transpose_pad_permute_cuda(v, vt, layout_flag)
+        v_fp8 = torch.empty(shape, dtype=torch.float8_e4m3fn, device=v.device)
+        v_scale = torch.empty((b, h, d), dtype=torch.float32, device=v.device)
+        if smooth_v:
+            vm = torch.empty((b, h, d), dtype=torch.float32, device=v.device)
+            _fused.mean_scale_fuse_quant_cuda(vt, v_fp8, vm, v_scale, n, scale_max, layout_flag)
+            return v_fp8, v_scale, vm
+        _fused.scale_fuse_quant_cuda(vt, v_fp8, v_scale, n, scale_max, layout_flag)
+        return v_fp8, v_scale, None
     if scale_max != 448.0:
         raise ValueError("per_channel_fp8: only scale_max=448.0 (the e4m3 maximum) is supported")
     b, h, n, d = _dims(v, tensor_layout)

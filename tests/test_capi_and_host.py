@@ -59,6 +59,13 @@ def test_c_abi_argument_errors_without_gpu():
     assert rc == L.PARO_ERR_INVALID_VALUE
     rc = lib.paro_quant_int8(p, 0, None, p, p, 1, 1, 64, 64, 0, 0, 64, 0, 0, 0, 0, 64, 0, 0, 32, 1, 0, 0.0, None)
     assert rc == L.PARO_ERR_RUNTIME and b"do not cover" in lib.paro_last_error()
+    rc = lib.paro_transpose_pad_permute(p, p, 0, 1, 1, 100, 64, 0, 0, 64, 0, 0, 64, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"ceil64(num_tokens) = 128" in lib.paro_last_error()
+    assert lib.paro_transpose_pad_permute(p, p, 0, 1, 1, 100, 80, 0, 0, 80, 0, 0, 128, None) == L.PARO_ERR_INVALID_VALUE
+    rc = lib.paro_channel_quant_fp8(p, 0, p, None, p, 1, 1, 64, 100, 64, 448.0, 0, 0, 64, 0, 0, 64, 0, 0, 0, 0, None)
+    assert rc == L.PARO_ERR_RUNTIME and b"shorter than ceil64" in lib.paro_last_error()
+    rc = lib.paro_channel_quant_fp8(p, 0, p, None, p, 1, 1, 64, 100, 128, 0.0, 0, 0, 128, 0, 0, 128, 0, 0, 0, 0, None)
+    assert rc == L.PARO_ERR_INVALID_VALUE and b"scale_max" in lib.paro_last_error()
     rc = lib.paro_permute_inv(p, p, 0, p, 1, 1, 100, 64, 10, 3, 5, 7, 0, 0, 64, 0, 0, 64, None)
     assert rc == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
     rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
@@ -91,8 +98,12 @@ def test_python_mirrors_reject_cpu_tensors_and_bad_flags():
         _qattn_sm80.qk_int8_sv_f16_accum_f16_attn(o, o, x, x, s, s, 1, 0, 2, 0.125, 0, torch.ones(1, 1, 1, 1, dtype=torch.bool))
     with pytest.raises(NotImplementedError):
         _qattn_sm80.qk_int4_sv_f16_accum_f16_attn()
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="Tensor input must be on CUDA"):
         _fused.transpose_pad_permute_cuda(x, x, 1)
+    with pytest.raises(RuntimeError, match="Tensor input must be on CUDA"):
+        _fused.mean_scale_fuse_quant_cuda(x, x, s, s, 64, 448.0, 1)
+    with pytest.raises(RuntimeError, match="Tensor input must be on CUDA"):
+        _fused.scale_fuse_quant_cuda(x, x, s, 64, 448.0, 1)
     with pytest.raises(AssertionError, match="must be on cuda"):
         core.paroattn_qk_int8_pv_fp16_cuda(x, x, x, torch.ones(1, 1, 1, dtype=torch.bool))
     with pytest.raises(RuntimeError):

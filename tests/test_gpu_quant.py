@@ -71,3 +71,59 @@ def test_sub_mean(dev):
     ref_vm = v.to(dev).mean(dim=2)
     ref = (v.to(dev) - ref_vm.unsqueeze(2)).to(torch.float16)  # bf16 subtraction, then fp16
     assert torch.equal(vs, ref)
+
+
+@pytest.mark.parametrize("layout,D,N,dtype", [("HND", 64, 200, torch.float16), ("NHD", 128, 333, torch.bfloat16),
+                                              ("HND", 128, 64, torch.float16), ("HND", 64, 17776, torch.bfloat16)])
+def test_reference_format_v_preparation(dev, layout, D, N, dtype):
+    """transpose_pad_permute_cuda, mean_scale_fuse_quant_cuda and scale_fuse_quant_cuda of
+    paroattention._fused (csrc/fused/pybind.cpp:29-33) against the oracle: the transposed, padded and
+    reordered tensor bit for bit; scales and means to fp32 summation order; codes equal except where the
+    mean's last bit moves a value across a rounding boundary."""
+    from paroatten_amd import _fused
+    B, H = 2, 3
+    g = torch.Generator().manual_seed(N + D)
+    v = (torch.randn(B, H, N, D, generator=g) * 1.5 + torch.randn(1, H, 1, D, generator=g)).to(dtype)
+    want_t = O.transpose_pad_permute(v)                               # [B,H,D,padded]
+    padded = want_t.shape[-1]
+    vd = v.to(dev)
+    flag = 1
+    if layout == "NHD":
+        vd = vd.transpose(1, 2).contiguous()                          # [B,N,H,D]
+        flag = 0
+        out = torch.full((B, D, H, padded), float("nan"), dtype=dtype, device=dev)
+    else:
+        out = torch.full((B, H, D, padded), float("nan"), dtype=dtype, device=dev)
+    _fused.transpose_pad_permute_cuda(vd, out, flag)
+    got_t = out.transpose(1, 2) if layout == "NHD" else out
+    assert torch.equal(got_t.cpu().view(torch.int16), want_t.view(torch.int16))
+    for smooth in (True, False):
+        codes = torch.zeros(out.shape, dtype=torch.float8_e4m3fn, device=dev)
+        scale = torch.empty(B, H, D, dtype=torch.float32, device=dev)
+        mean = torch.empty(B, H, D, dtype=torch.float32, device=dev)
+        if smooth:
+            _fused.mean_scale_fuse_quant_cuda(out, codes, mean, scale, N, 448.0, flag)
+        else:
+            _fused.scale_fuse_quant_cuda(out, codes, scale, N, 448.0, flag)
+        wc, ws, wm = O.channel_quant_fp8(want_t, N, sub_mean=smooth)
+        gc = (codes.transpose(1, 2) if layout == "NHD" else codes).cpu().view(torch.uint8)
+        assert torch.allclose(scale.cpu(), ws, rtol=2e-6, atol=0)
+        if smooth:
+            assert torch.allclose(mean.cpu(), wm, rtol=1e-5, atol=1e-6)
+        diff = (gc.int() - wc.view(torch.uint8).int()).abs()
+        assert int(diff.max()) <= 1 and float((diff != 0).float().mean()) <= (1e-3 if smooth else 0.0)
+
+
+def test_per_channel_fp8_reference_order(dev):
+    """quant.per_channel_fp8(tile_order=False) = the reference's own sequence of the three calls
+    (paroattention/quant.py:266-293)"""
+    g = torch.Generator().manual_seed(9)
+    v = torch.randn(1, 2, 150, 64, generator=g).to(torch.float16)
+    v8, vs, vm = _q().per_channel_fp8(v.to(dev), tile_order=False)
+    assert v8.shape == (1, 2, 64, 192) and v8.dtype == torch.float8_e4m3fn
+    wc, ws, wm = O.channel_quant_fp8(O.transpose_pad_permute(v), 150)
+    assert torch.allclose(vs.cpu(), ws, rtol=2e-6) and torch.allclose(vm.cpu(), wm, rtol=1e-5, atol=1e-6)
+    diff = (v8.cpu().view(torch.uint8).int() - wc.view(torch.uint8).int()).abs()
+    assert int(diff.max()) <= 1 and float((diff != 0).float().mean()) <= 1e-3
+    v8n, vsn, none = _q().per_channel_fp8(v.to(dev), smooth_v=False, tile_order=False, scale_max=224.0)
+    assert none is None and torch.allclose(vsn.cpu(), v.float().abs().amax(dim=2) / 224.0, rtol=2e-6)

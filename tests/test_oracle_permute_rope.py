@@ -95,3 +95,49 @@ def test_per_channel_fp8_against_library_cast():
     rel = (deq - centred).abs() / centred.abs().clamp_min(1e-3)
     assert float(rel.max()) <= 0.0625 + 1e-3 or float(((deq - centred).abs()).max()) < 2e-2  # 3 mantissa bits
     assert float(v8.float().abs().max()) == 448.0
+
+
+def test_transpose_pad_permute_order_is_stated_twice_by_the_reference():
+    """the kernel's formula (fused.cu:287-291) and the docstring's literal list (quant.py:231-234) agree,
+    and the oracle is torch.transpose + pad with that order"""
+    for r in range(16):
+        assert O.V_SHUFFLE16[O.shuffle16_position_of(r)] == r
+    assert sorted(O.V_SHUFFLE16) == list(range(16))
+    g = torch.Generator().manual_seed(0)
+    v = torch.randn(2, 3, 100, 64, generator=g).to(torch.float16)
+    out = O.transpose_pad_permute(v)
+    assert out.shape == (2, 3, 64, 128) and (out[..., 112:] == 0).all()
+    for n in (0, 1, 2, 8, 17, 50, 99):
+        pos = (n // 16) * 16 + O.shuffle16_position_of(n % 16)
+        assert torch.equal(out[..., pos], v[:, :, n, :])
+    # tokens 100..111 share a group of 16 with real tokens: zero, at their shuffled positions
+    assert (out[..., [96 + O.shuffle16_position_of(r) for r in range(4, 16)]] == 0).all()
+
+
+def test_channel_quant_fp8_reduces_to_per_channel_fp8_and_keeps_the_quirk():
+    g = torch.Generator().manual_seed(1)
+    v = (torch.randn(1, 2, 128, 64, generator=g) + 0.7).to(torch.bfloat16)
+    x = v.transpose(2, 3).contiguous()
+    codes, sc, mean = O.channel_quant_fp8(x, 128)
+    v8, vs, vm = O.per_channel_fp8(v)            # pinned by its own tests
+    assert torch.allclose(mean, vm, atol=1e-6) and torch.allclose(sc, vs, rtol=1e-5)
+    same = (codes.view(torch.uint8) == v8.transpose(2, 3).view(torch.uint8)).float().mean()
+    assert same >= 0.999                          # a last-bit difference of the mean flips a tie here and there
+    # 100 real tokens in rows padded to 128: statistics over the first 112, mean divides by 112
+    xp = x.clone()
+    xp[..., 100:] = 0
+    codes, sc, mean = O.channel_quant_fp8(xp, 100)
+    assert codes.shape[-1] == 128
+    assert torch.allclose(mean, xp[..., :100].float().sum(-1) / 112, atol=1e-6)
+    cen = xp[..., :112].float() - mean[..., None]
+    assert torch.allclose(sc, cen.abs().amax(-1) / 448.0, rtol=1e-6)
+    deq = codes.float() * sc[..., None] + mean[..., None]
+    assert ((deq - xp.float()).abs() <= sc[..., None] * 16.0 + 1e-6).all()     # half the widest e4m3 cell
+    assert (codes.float().abs().amax(-1) == 448.0).all()                          # the extreme maps to +-448
+    # without the mean: symmetric scale, zeros stay zero codes
+    codes, sc, none = O.channel_quant_fp8(xp, 100, sub_mean=False)
+    assert none is None and torch.allclose(sc, xp[..., :112].float().abs().amax(-1) / 448.0, rtol=1e-6)
+    assert (codes[..., 100:].float() == 0).all()
+    # a constant row gives zero codes, not NaN
+    codes, sc, mean = O.channel_quant_fp8(torch.full((1, 1, 2, 64), 3.0, dtype=torch.float16), 64)
+    assert (codes.float() == 0).all() and (sc == 0).all() and torch.allclose(mean, torch.full((1, 1, 2), 3.0))
