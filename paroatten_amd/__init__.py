@@ -19,12 +19,25 @@ from .wan import PARO_WanAttnProcessor, PARO_WanAttnProcessor2_0, set_paro_proce
 
 __all__ = ["paroattn", "paroattn_qk_int8_pv_fp16_cuda", "PARO_CogVideoXAttnProcessor2_0",
            "PARO_CogVideoXAttnProcessor", "PARO_WanAttnProcessor2_0", "PARO_WanAttnProcessor",
-           "set_paro_processors", "install_alias"]
+           "set_paro_processors", "install_alias", "compiled_extension"]
 
 
-def install_alias(name: str = "paroattention"):
+def compiled_extension():
+    """The PyTorch-ROCm C++ extension (csrc/torch_binding.cpp -> paroatten_amd/_ext.so): submodules
+    `_qattn_sm80`, `_fused`, `_rope` with the reference's positional pybind signatures, bound to the same
+    C ABI as the ctypes mirrors of this package.  Raises ImportError if it has not been built."""
+    try:
+        from . import _ext
+    except ImportError as e:   # pragma: no cover - depends on the build
+        raise ImportError(f"paroatten_amd/_ext.so is not built: run `python paroatten_amd/build.py` ({e})") from e
+    return _ext
+
+
+def install_alias(name: str = "paroattention", compiled: bool = False):
     """Make `import paroattention`, `paroattention.core`, `paroattention._qattn_sm80`, ... resolve to
-    this package."""
+    this package.  With compiled=True the three extension-module names resolve to the compiled C++
+    extension instead of the ctypes mirrors (same C ABI underneath, the reference's exact signatures, no
+    extra keywords)."""
     pkg = sys.modules[__name__]
     sys.modules[name] = pkg
     for sub in list(sys.modules):
@@ -33,4 +46,8 @@ def install_alias(name: str = "paroattention"):
     # the reference keeps the Wan twin of prefetch_utils in its own module (paroattention/prefetch_wan.py)
     sys.modules[name + ".prefetch_wan"] = prefetch_utils
     pkg.prefetch_wan = prefetch_utils
+    if compiled:
+        ext = compiled_extension()
+        for sub in ("_qattn_sm80", "_fused", "_rope"):
+            sys.modules[f"{name}.{sub}"] = getattr(ext, sub)
     return pkg

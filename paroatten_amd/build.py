@@ -1,4 +1,5 @@
-"""Build libparoatten_hip.so (device code for gfx950 only) with hipcc, in-tree.
+"""Build libparoatten_hip.so (device code for gfx950 only) with hipcc, and the PyTorch-ROCm C++
+extension paroatten_amd/_ext.so (host code only, binds the library's C ABI) with g++, both in-tree.
 
     python paroatten_amd/build.py
 
@@ -59,6 +60,33 @@ def _compile(src: str, verbose: bool) -> Path:
     return obj
 
 
+EXT = PKG / "_ext.so"
+
+
+def build_ext(verbose: bool = False) -> Path:
+    """Compile csrc/torch_binding.cpp (pybind11 + torch headers, no device code) into
+    paroatten_amd/_ext.so, linked against libparoatten_hip.so ($ORIGIN/lib) and torch's libraries."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = Path(torch.__file__).resolve().parent / "lib"
+    inc = [*ce.include_paths("cuda"), sysconfig.get_paths()["include"], str(PKG.parent / "include")]
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_ext",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-Wno-deprecated-declarations",
+           *[f"-I{i}" for i in inc], str(CSRC / "torch_binding.cpp"), "-o", str(EXT),
+           f"-L{tlib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+           f"-L{LIBDIR}", "-lparoatten_hip", "-Wl,-rpath,$ORIGIN/lib", f"-Wl,-rpath,{tlib}"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"g++ failed on torch_binding.cpp:\n{r.stdout}\n{r.stderr}")
+    if verbose and r.stderr.strip():
+        print(r.stderr, file=sys.stderr)
+    return EXT
+
+
 def build(force: bool = True, verbose: bool = False) -> Path:
     """Compile every HIP source and link the shared library.  Always compiles when force."""
     LIBDIR.mkdir(exist_ok=True)
@@ -78,3 +106,5 @@ def build(force: bool = True, verbose: bool = False) -> Path:
 if __name__ == "__main__":
     path = build(force="--force" in sys.argv or True, verbose=True)
     print(path)
+    if "--no-ext" not in sys.argv:
+        print(build_ext(verbose=True))
