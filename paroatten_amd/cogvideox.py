@@ -68,6 +68,7 @@ class _ParoProcessorBase:
         self.call_count = 0
         self._orders_cache = {}
         self._table_cache = (None, None, None)
+        self._table_src = None
         self.i_timestep = 0
         self.i_block = 0
 
@@ -86,18 +87,42 @@ class _ParoProcessorBase:
         ps = getattr(self, "prefetch_stream", None)
         if ps is not None:
             return ps.mask_for(self.i_timestep, self.i_block)
-        m = self.sparse_mask[self.i_timestep, self.i_block]
+        # the callback's value after the last denoising step is T (prefetch_utils.py:22-25): clamp as the
+        # prefetch stream does
+        t = min(max(int(self.i_timestep), 0), self.sparse_mask.shape[0] - 1)
+        m = self.sparse_mask[t, self.i_block]
         if m.dtype != torch.bool:
             m = m.bool()
         return m
 
     def _grid_for(self, n_img: int, known) -> Tuple[int, int, int]:
+        """(F, H, W) of the latent grid.  A token count does not determine it (21*30*52 = 21*52*30: a
+        portrait video has the same count as a landscape one), so the `grid` given to the processor
+        wins; without it the model's default landscape grid is assumed for a known token count, as
+        the reference hard-codes it (cogvideox.py:31-33, wan.py:33-35), with a warning the first time."""
         g = self.grid
         if g is None:
             g = known.get(n_img)
+            if g is not None and not getattr(self, "_grid_warned", False):
+                import warnings
+                warnings.warn(f"PARO processor: no grid given, assuming (F, H, W) = {g} for {n_img} image tokens; "
+                              "pass grid=(F, H, W) if the latent has another orientation", stacklevel=3)
+                self._grid_warned = True
         if g is None or g[0] * g[1] * g[2] != n_img:
             raise ValueError(f"{n_img} image tokens do not match grid {g}: set the processor's `grid` to (F, H, W)")
         return g
+
+    def _same_source(self, src) -> bool:
+        """True if `src` (a tensor or a tuple of tensors) is what the cached tables were made from: the
+        very same tensor objects, unmodified since.  An address alone would not do: a rotary table that
+        the model rebuilds on every forward can come back at a recycled address with other contents."""
+        old = self._table_src
+        if old is None or len(old) != len(src):
+            return False
+        return all(t is o and t._version == v for t, (o, v) in zip(src, old))
+
+    def _remember_source(self, src):
+        self._table_src = [(t, t._version) for t in src]
 
     @staticmethod
     def _rope_permute(query, key, value, orders, grid, n_text, cos, sin, rotate_key=True):
@@ -143,10 +168,10 @@ class PARO_CogVideoXAttnProcessor2_0(_ParoProcessorBase):
 
     def _tables(self, image_rotary_emb, device):
         cos, sin = image_rotary_emb
-        key = (cos.data_ptr(), sin.data_ptr(), str(device))
-        if self._table_cache[0] != key:
-            self._table_cache = (key, cos.to(device=device, dtype=torch.float32).contiguous(),
+        if self._table_cache[0] != str(device) or not self._same_source((cos, sin)):
+            self._table_cache = (str(device), cos.to(device=device, dtype=torch.float32).contiguous(),
                                  sin.to(device=device, dtype=torch.float32).contiguous())
+            self._remember_source((cos, sin))
         return self._table_cache[1], self._table_cache[2]
 
     def __call__(self, attn, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,

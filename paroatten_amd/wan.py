@@ -43,12 +43,12 @@ def permute_attn_out(attn_out, permute_plan, i_block, grid=(21, 45, 80), n_text=
 
 class PARO_WanAttnProcessor2_0(_ParoProcessorBase):
     def _tables(self, rotary_emb, device, head_dim):
-        key = (rotary_emb.data_ptr(), str(device))
-        if self._table_cache[0] != key:
+        if self._table_cache[0] != str(device) or not self._same_source((rotary_emb,)):
             freqs = rotary_emb.reshape(-1, head_dim // 2)
             cos, sin = rope.complex_to_real_tables(freqs)
-            self._table_cache = (key, cos.to(device=device, dtype=torch.float32).contiguous(),
+            self._table_cache = (str(device), cos.to(device=device, dtype=torch.float32).contiguous(),
                                  sin.to(device=device, dtype=torch.float32).contiguous())
+            self._remember_source((rotary_emb,))
         return self._table_cache[1], self._table_cache[2]
 
     def __call__(self, attn, hidden_states: torch.Tensor, encoder_hidden_states: Optional[torch.Tensor] = None,

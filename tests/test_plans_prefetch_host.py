@@ -81,3 +81,30 @@ def test_pack_mask_bits_matches_numpy(n):
     # element 8j+i is bit i of byte j
     j, i = (n - 1) // 8, (n - 1) % 8
     assert bool((int(bits[0, j]) >> i) & 1) == bool(m[0, n - 1])
+
+
+def test_processor_grid_and_table_cache_rules():
+    """a token count does not fix (F,H,W): the explicit grid wins, a guessed one warns once; the
+    rotary-table cache is keyed on the identity and version of the source tensors, not on an address"""
+    from paroatten_amd.cogvideox import PARO_CogVideoXAttnProcessor2_0
+    from paroatten_amd.wan import WAN_GRIDS, PARO_WanAttnProcessor2_0
+    p = PARO_WanAttnProcessor2_0(grid=(21, 52, 30))
+    assert p._grid_for(21 * 30 * 52, WAN_GRIDS) == (21, 52, 30)            # portrait: as given
+    q = PARO_WanAttnProcessor2_0()
+    with pytest.warns(UserWarning, match="assuming"):
+        assert q._grid_for(21 * 30 * 52, WAN_GRIDS) == (21, 30, 52)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        assert q._grid_for(21 * 30 * 52, WAN_GRIDS) == (21, 30, 52)        # only once
+    with pytest.raises(ValueError):
+        PARO_WanAttnProcessor2_0(grid=(21, 30, 52))._grid_for(100, WAN_GRIDS)
+    c = PARO_CogVideoXAttnProcessor2_0()
+    cos, sin = torch.zeros(8, 4, dtype=torch.float64), torch.ones(8, 4, dtype=torch.float64)   # converted: a copy
+    a1 = c._tables((cos, sin), "cpu")
+    assert c._tables((cos, sin), "cpu")[0] is a1[0]                        # same objects, unmodified: cached
+    cos.add_(1.0)                                                          # modified in place: rebuilt
+    a2 = c._tables((cos, sin), "cpu")
+    assert a2[0] is not a1[0] and torch.equal(a2[0], cos.float())
+    cos2 = cos.clone()                                                     # another object: rebuilt
+    assert c._tables((cos2, sin), "cpu")[0] is not a2[0]
