@@ -39,6 +39,12 @@ PEAK_MFMA_TOPS = 5000.0  # dense INT8 / FP8 MFMA peak of MI355X, TOP/s
 PEAK_HBM_GBS = 8000.0
 HEADLINE_DENSITY = 0.3
 DENSITIES = (0.5, 0.3, 0.2)
+# per workload: (headline density, densities reported), as the benchmark list states them
+WORKLOAD_DENSITIES = {
+    "cogvideox5b": (0.3, (0.5, 0.3, 0.2)),
+    "wan14b_480p": (0.3, (0.3,)),
+    "wan14b_720p": (0.2, (0.2, 1.0)),     # 1.0 = the dense comparison run
+}
 # HBM bytes per attention-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/path_kernels_cogvideox5b_hbm_traffic.txt): FETCH_SIZE 166963 x 2.0 KiB + WRITE_SIZE 213836 x 1.0 KiB,
 # the factors being what the same counters read for a plain copy of known size; the same at every density
@@ -73,12 +79,42 @@ def event_time_ms(fn, reps, warmup):
     return e0.elapsed_time(e1) / reps
 
 
+def cpu_model_name():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_cfg0_whole_path(threads):
+    """Benchmark configuration 0 in full on the CPU oracle: B=1, H=2, D=64, fp16, 16x16x16 grid (N=4096),
+    K bias, density 0.5, per-head permutation -> INT8 (K smoothed) -> block-sparse attention -> inverse
+    permutation."""
+    from oracle import paro_oracle as O
+    from paroatten_amd import synth
+
+    wl = synth.WORKLOADS["cfg0_plumbing"]
+    q, k, v = synth.make_qkv(wl.B, wl.H, wl.N, wl.D, wl.dtype, seed=0)
+    mask = synth.make_block_mask(wl.H, wl.nb, 0.5, seed=1)[None]
+    plan = synth.make_permute_plan(1, wl.H, seed=2)
+    t0 = time.perf_counter()
+    O.paro_path(q, k, v, mask, plan, 0, wl.grid, wl.n_text)
+    dt = time.perf_counter() - t0
+    return {"seconds": round(dt, 3), "dense_equiv_tops": synth.dense_equiv_ops(wl.B, wl.H, wl.N, wl.D) / dt / 1e12,
+            "threads": threads}
+
+
 def cpu_baseline(wl, density, heads=16, threads=None):
     """The oracle (CPU port of the reference path) on a slice: B=1, `heads` heads, full N."""
     from oracle import paro_oracle as O
     from paroatten_amd import synth
 
-    threads = threads or min(16, os.cpu_count() or 1)
+    host_cores = os.cpu_count() or 1
+    threads = threads or min(16, host_cores)   # the share of the host one GPU job is given
     torch.set_num_threads(threads)
     N, D = wl.N, wl.D
     q, k, v = synth.make_qkv(1, heads, N, D, wl.dtype, seed=7)
@@ -93,11 +129,14 @@ def cpu_baseline(wl, density, heads=16, threads=None):
         "value": ops / dt / 1e12,
         "unit": "TOPS (dense-equivalent 4*B*H*D*N^2/t)",
         "cores": threads,
+        "host_logical_cores": host_cores,
+        "cpu_model": cpu_model_name(),
         "kind": "port",
         "sample": f"oracle quant + block-sparse attention, B=1, {heads} of {wl.B * wl.H} (batch, head) pairs, "
                   f"N={N}, D={D}, density {density}, {dt:.1f} s; per-head work is independent, so the "
                   f"whole workload would take about {dt * wl.B * wl.H / heads:.0f} s",
         "seconds": dt,
+        "cfg0_whole_path": cpu_cfg0_whole_path(threads),
     }
 
 
@@ -110,7 +149,17 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="only the headline density and the attention kernel: the run to put under a profiler")
     ap.add_argument("--workload", default="cogvideox5b", choices=["cogvideox5b", "wan14b_480p", "wan14b_720p"])
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="attention kernel on all-zero q8 / k8 / v8 (same masks, same instruction stream, no data "
+                         "toggling): with a profiler's GRBM_GUI_ACTIVE this separates what the shader clock does "
+                         "under the kernel from what its instruction mix costs.  Not a benchmark result.")
+    ap.add_argument("--pacing", choices=["auto", "on", "off"], default="auto",
+                    help="attention launch: generation-paced resident workgroups (on), the plain launch (off), or the "
+                         "library's own choice (auto: paced when one head's K8+V8 exceed an XCD's L2)")
+    ap.add_argument("--exact-exp", action="store_true", help="attention kernel with exact exponentials (flag PARO_ATTN_EXACT_EXP)")
     args = ap.parse_args()
+    if args.pacing != "auto":   # the library's default for calls that carry neither pacing flag
+        os.environ["PARO_ATTN_PACING"] = "1" if args.pacing == "on" else "0"
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU (every kernel of the path is independent per "
               "(batch, head); nothing here uses a second GPU). Run with --gpus 1.", file=sys.stderr)
@@ -129,6 +178,8 @@ def main():
     torch.cuda.set_device(dev)
     lib = L.load()
     wl = synth.WORKLOADS[args.workload]
+    global HEADLINE_DENSITY, DENSITIES
+    HEADLINE_DENSITY, DENSITIES = WORKLOAD_DENSITIES[args.workload]
     B, H, D, N, nb = wl.B, wl.H, wl.D, wl.N, wl.nb
     sm_scale = D ** -0.5
 
@@ -146,20 +197,26 @@ def main():
     q8, qs, k8, ks = Q.per_warp_int8(qp, kp, km, BLKQ=64, WARPQ=32, BLKK=64)
     out = torch.empty_like(q)
     ws = torch.empty(qattn.workspace_bytes(B, H, N, D), dtype=torch.uint8, device=dev)
-    masks = {d: synth.make_block_mask(H, nb, d, seed=3, device=dev) for d in DENSITIES}
+    masks = {d: (synth.make_block_mask(H, nb, d, seed=3, device=dev) if d < 1.0
+                 else torch.ones(H, nb, nb, dtype=torch.bool, device=dev)) for d in DENSITIES}
     dense_ops = synth.dense_equiv_ops(B, H, N, D)
 
     def entry(mask):  # the reference's extension entry point: V fp16 in, O out
         qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, vp, out, qs, ks, 1, 0, 2, sm_scale, 0, mask, workspace=ws)
 
     v8, vsc, vm = Q.per_channel_fp8(vp)
+    if args.zero_operands:
+        aq8, ak8, av8 = torch.zeros_like(q8), torch.zeros_like(k8), torch.zeros_like(v8)
+    else:
+        aq8, ak8, av8 = q8, k8, v8
+    attn_flags = L.PARO_ATTN_EXACT_EXP if args.exact_exp else 0
 
     def attn_only(mask):  # the attention kernel alone (for the roofline)
         L.check(lib.paro_attn_sparse_fwd(
-            L.ptr(q8), L.ptr(k8), L.ptr(v8), L.ptr(qs), L.ptr(ks), L.ptr(vsc), L.ptr(vm), L.ptr(mask), 0,
+            L.ptr(aq8), L.ptr(ak8), L.ptr(av8), L.ptr(qs), L.ptr(ks), L.ptr(vsc), L.ptr(vm), L.ptr(mask), 0,
             L.ptr(out), L.DTYPE_CODE[out.dtype], None, None, B, H, H, N, N, D,
             q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
-            out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, 0, L.stream_of(out)))
+            out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, attn_flags, L.stream_of(out)))
 
     # ---- the timed region: exactly K steps between synchronisations -------------------------
     head_mask = masks[HEADLINE_DENSITY]
@@ -175,7 +232,9 @@ def main():
     value = dense_ops / (ms_per_step * 1e-3) / 1e12
 
     # ---- per-density detail and the roofline of the attention kernel -------------------------
-    reps = max(5, min(args.steps, 50))
+    # at least 100 repetitions per figure whatever --steps says (the reference's own benchmark takes 100,
+    # bench/bench.py:74-76), fewer only for launches of tens of milliseconds
+    reps = max(100, args.steps) if args.workload != "wan14b_720p" else max(20, min(args.steps, 100))
     dens = {}
     for d in ((HEADLINE_DENSITY,) if args.headline_only else DENSITIES):
         t_entry = event_time_ms(lambda: entry(masks[d]), reps, 2)
@@ -210,7 +269,7 @@ def main():
         "bound": "mfma",
         "achieved": achieved,
         "peak": PEAK_MFMA_TOPS,
-        "unit": "TFLOP/s",
+        "unit": "TOP/s",
         "frac": round(achieved / PEAK_MFMA_TOPS, 4),
         "traffic": ATTN_TRAFFIC_BYTES if args.workload == "cogvideox5b" else None,
         "ops_per_launch": hk["kept_blocks"] * 4.0 * 64 * 64 * D,
@@ -283,6 +342,8 @@ def main():
             "density": HEADLINE_DENSITY,
         },
         "pct_mfma_peak": hk["pct_mfma_peak_kernel"],
+        "attention_operands": "all zero (--zero-operands: a clock experiment, not a result)" if args.zero_operands else "synthetic",
+        "reps_per_figure": reps,
         "densities": dens,
         "path": path,
         "roofline": roofline,

@@ -20,6 +20,8 @@ PARO_ERR_RUNTIME = -2
 PARO_ERR_UNSUPPORTED = -3
 PARO_ERR_HIP = -4
 PARO_ATTN_EXACT_EXP = 1
+PARO_ATTN_PACED = 2
+PARO_ATTN_UNPACED = 4
 
 DTYPE_CODE = {torch.float16: 0, torch.bfloat16: 1}
 

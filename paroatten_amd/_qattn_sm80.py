@@ -11,6 +11,8 @@ Differences, all relaxations or added checks:
   * `value` may be float16 (as in the reference) or bfloat16 (saves the caller's `.to(float16)`);
   * keyword `exact_exp=True` evaluates the softmax exponentials in fp32 before the FP8 rounding instead
     of building the e4m3 byte directly (slower, slightly more accurate; always on with return_lse);
+  * keyword `pacing=True/False` picks the launch form of the attention kernel (see PARO_ATTN_PACED in
+    include/paroatten.h; bit-identical results), None leaves it to the library;
   * `sparse` IS validated (the reference reads it through a raw pointer unchecked): bool or uint8,
     on the GPU, contiguous, shape [B,H,nbq,nbk] or [H,nbq,nbk] (shared by the batch);
   * the INT4 and INT8-P.V variants registered by the reference are experimental prototypes with
@@ -29,13 +31,22 @@ def _chk(cond, msg):
         raise RuntimeError(msg)
 
 
+def _flags(exact_exp, pacing):
+    """pacing: None (the library chooses), True (PARO_ATTN_PACED) or False (PARO_ATTN_UNPACED): the launch
+    form only, results are bit-identical."""
+    f = _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0
+    if pacing is not None:
+        f |= _lib.PARO_ATTN_PACED if pacing else _lib.PARO_ATTN_UNPACED
+    return f
+
+
 def workspace_bytes(B, Hkv, Nk, D):
     return int(load().paro_attn_workspace_bytes(B, Hkv, Nk, D))
 
 
 def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_scale, tensor_layout, is_causal,
                                   qk_quant_gran, sm_scale, return_lse, sparse, *, smooth_v=True, exact_exp=False,
-                                  workspace=None):
+                                  workspace=None, pacing=None):
     for t, n in ((query, "query"), (key, "key"), (value, "value"), (output, "output"),
                  (query_scale, "query_scale"), (key_scale, "key_scale")):
         _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
@@ -116,12 +127,12 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
         value.stride(0), value.stride(sh), value.stride(sn),
         output.stride(0), output.stride(sh), output.stride(sn),
         tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0,
-        _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0, stream_of(query))
+        _flags(exact_exp, pacing), stream_of(query))
     return lse
 
 
 def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_scale, sm_scale, sparse,
-                          is_causal=0, return_lse=0, exact_exp=False, unpermute=None):
+                          is_causal=0, return_lse=0, exact_exp=False, unpermute=None, pacing=None):
     """The attention kernel alone, on operands that are already in its formats (HND, contiguous):
     q8/k8 int8 [B,H,N,D] / [B,Hkv,Nk,D], v8 = FP8 tiles from paro_v_fp8_pack or the fused
     preparation, v_scale / v_mean f32 [B,Hkv,D] (v_mean None: V was not mean-smoothed).  No
@@ -154,7 +165,7 @@ def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_
         _chk(tuple(sparse.shape) == (H, nbq, nbk), f"Tensor sparse must have shape ([{B},] {H}, {nbq}, {nbk})")
         sparse_bs = 0
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q8.device) if return_lse else torch.empty(0)
-    flags = _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0
+    flags = _flags(exact_exp, pacing)
     strides = (q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
                output.stride(0), output.stride(1), output.stride(2))
     if unpermute is None:

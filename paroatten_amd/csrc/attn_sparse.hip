@@ -28,6 +28,8 @@
 // scale indexing :100-133, mask indexing :222/:268, out-of-range columns attn_utils.cuh:355-381,
 // softmax recurrence attn_utils.cuh:383-488, normalisation :786-840, lse = log2(d) + m (:711-723).
 #include "paro_device.hpp"
+#include <mutex>
+#include <stdlib.h>
 #include <type_traits>
 
 namespace paro {
@@ -55,6 +57,7 @@ struct AttnParams {
   // n_text + unpermute(r - n_text, orders[h]) (rows below n_text stay); orders == nullptr: row r
   const int* orders;
   int n_text, F, Hh, W;
+  int pacing;  // +1: paced launch asked for, -1: plain launch asked for, 0: the library chooses
 };
 
 // P~ = 2^(S*c - m + P_EXP_OFFSET).  m is the running row maximum, refreshed lazily: only when a
@@ -151,8 +154,9 @@ __device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, u
 // Waves per SIMD the register budget is set for: the D = 64 production variants fit 168 registers.
 #define PARO_ATTN_WAVES_PER_SIMD ((D == 64 && !CAUSAL && !DUMP && !LSE) ? 3 : 2)
 
+// One 64-row q-block `vid` (numbered over batch, head, q-block) by one workgroup of two waves.
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
-__global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_kernel(const AttnParams p) {
+__device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) {
   using Lds = AttnLds<D>;
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
   constexpr int DT_TILES = D / 32;  // 32-channel tiles of O^T
@@ -167,10 +171,6 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  // XCD-aware renumbering: hardware deals workgroup ids round-robin to the 8 XCDs
-  const int per = gridDim.x >> 3;
-  const int vid = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-  if (vid >= p.total) return;
   const int qb = vid % p.nbq;
   const int bh = vid / p.nbq;
   const int h = bh % p.H, b = bh / p.H;
@@ -679,9 +679,107 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
 }
 
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
+__global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_kernel(const AttnParams p) {
+  // XCD-aware renumbering: hardware deals workgroup ids round-robin to the 8 XCDs
+  const int per = gridDim.x >> 3;
+  const int vid = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+  if (vid >= p.total) return;
+  attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>(p, vid);
+}
+
+// The same work with a resident set of workgroups per XCD that take the XCD's q-blocks generation by
+// generation: all of them start a q-block together and so walk the key blocks of the head roughly in step.
+// For heads whose K8 + V8 exceed the XCD's L2 (Wan 720p: 19 MB against 4 MB): in the ordinary launch
+// the workgroups of an XCD sit at unrelated positions of the key sequence, the L2 sees a uniform stream
+// over the whole head and hits at (L2 size / head size); started together, neighbours in time are
+// neighbours in the key sequence.  The meeting point between generations only paces: a workgroup that
+// has waited `spin_limit` rounds goes on regardless, so the kernel finishes whatever the residency or
+// the state of the counters (they are zeroed by a small launch in front of this one).
+constexpr int PACE_PAD = 32;   // counters 128 bytes apart: one per XCD
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
+__global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
+    attn_sparse_paced_kernel(const AttnParams p, unsigned* __restrict__ counters, const int per, const int spin_limit) {
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, G = gridDim.x >> 3;
+  const int first = xcd * per, last = min(first + per, p.total);
+  unsigned arrivals = 0;
+  for (int base = first; base < last; base += G) {
+    const int vid = base + slot;
+    if (vid < last) attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>(p, vid);
+    if (base + G >= last) break;
+    // every workgroup of the XCD arrives once per generation, with or without a q-block of its own
+    __syncthreads();   // also: both waves are done with this q-block's lists in LDS
+    if (threadIdx.x == 0) {
+      arrivals += (unsigned)G;
+      unsigned* c = counters + xcd * PACE_PAD;
+      __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int spin = 0; spin < spin_limit; spin++) {
+        if (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= arrivals) break;
+        __builtin_amdgcn_s_sleep(32);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+__global__ void attn_pace_reset_kernel(unsigned* counters) { counters[threadIdx.x] = 0u; }
+
+// counters of the paced kernel: library-owned, one set per GPU (looked up once per device)
+static __device__ __align__(256) unsigned g_pace_counters[8 * PACE_PAD];
+constexpr int PACE_MAX_DEVICES = 64;
+struct PaceDevice { unsigned* counters; int cus; };
+static PaceDevice g_pace_dev[PACE_MAX_DEVICES];
+static std::mutex g_pace_mu;
+
+static int pace_device(PaceDevice* out) {
+  int dev = -1;
+  PARO_HIP(hipGetDevice(&dev));
+  PARO_CHECK(dev >= 0 && dev < PACE_MAX_DEVICES, PARO_ERR_RUNTIME, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_pace_mu);
+  if (g_pace_dev[dev].counters == nullptr) {
+    void* ptr = nullptr;
+    PARO_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_pace_counters)));
+    int cus = 0;
+    PARO_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    g_pace_dev[dev].cus = cus;
+    g_pace_dev[dev].counters = static_cast<unsigned*>(ptr);
+  }
+  *out = g_pace_dev[dev];
+  return PARO_OK;
+}
+
+// The caller's flags decide (PARO_ATTN_PACED / PARO_ATTN_UNPACED); without either, the environment
+// variable PARO_ATTN_PACING (0: never, 1: always) does, and without that the launch is paced when one
+// head's K8 + V8 exceed the 4 MB L2 of an XCD.  PARO_ATTN_PACE_SPINS: rounds (about 1 us each) a workgroup
+// waits for its generation at most (default 4096).
+static bool want_pacing(const AttnParams& p, int D) {
+  if (p.pacing != 0) return p.pacing > 0;
+  if (const char* e = getenv("PARO_ATTN_PACING")) return e[0] == '1';
+  return (int64_t)p.nbk * 64 * D * 2 > (int64_t)4 << 20;
+}
+
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
-  const int grid = ((p.total + 7) / 8) * 8;
   const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + AttnLds<D>::LIST_PAD) * 6 + 15) & ~(size_t)15);
+  if (!DUMP && want_pacing(p, D)) {
+    auto kern = attn_sparse_paced_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
+    if (smem > 48 * 1024)
+      PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    PaceDevice pd;
+    if (int rc = pace_device(&pd)) return rc;
+    int per_cu = 0;
+    PARO_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, 128, smem));
+    const int G = per_cu * (pd.cus / 8);        // workgroups resident on one XCD
+    const int per = (p.total + 7) / 8;          // q-blocks per XCD, a contiguous range of (batch, head, q-block)
+    if (G > 0 && per > G) {                     // more than one generation: otherwise the plain launch is the same
+      int spins = 4096;
+      if (const char* e = getenv("PARO_ATTN_PACE_SPINS")) spins = atoi(e);
+      hipLaunchKernelGGL(attn_pace_reset_kernel, dim3(1), dim3(8 * PACE_PAD), 0, st, pd.counters);
+      hipLaunchKernelGGL(kern, dim3(8 * G), dim3(128), smem, st, p, pd.counters, per, spins);
+      PARO_HIP(hipGetLastError());
+      return PARO_OK;
+    }
+  }
+  const int grid = ((p.total + 7) / 8) * 8;
   auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
   if (smem > 48 * 1024)
     PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -717,7 +815,9 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
                             int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
                             int64_t o_stride_n, float sm_scale, int is_causal, int flags, const int32_t* orders,
                             int n_text, int F, int Hh, int W, void* stream) {
-  PARO_CHECK((flags & ~PARO_ATTN_EXACT_EXP) == 0, PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
+  PARO_CHECK((flags & ~(PARO_ATTN_EXACT_EXP | PARO_ATTN_PACED | PARO_ATTN_UNPACED)) == 0 &&
+                 (flags & (PARO_ATTN_PACED | PARO_ATTN_UNPACED)) != (PARO_ATTN_PACED | PARO_ATTN_UNPACED),
+             PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
   PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && v_scale && sparse && out, PARO_ERR_RUNTIME,
              "paro_attn_sparse_fwd: null tensor pointer");
   PARO_CHECK(B > 0 && H > 0 && Hkv > 0 && Nq > 0 && Nk > 0, PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: empty shape");
@@ -759,6 +859,7 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
   p.total = B * H * nbq;
   p.sm_scale_log2e = sm_scale * 1.4426950408889634f;
   p.orders = orders; p.n_text = n_text; p.F = F; p.Hh = Hh; p.W = W;
+  p.pacing = (flags & PARO_ATTN_PACED) ? 1 : ((flags & PARO_ATTN_UNPACED) ? -1 : 0);
   hipStream_t st = (hipStream_t)stream;
   const bool dump = s_dump != nullptr;
   const bool exact = (flags & PARO_ATTN_EXACT_EXP) != 0;

@@ -256,3 +256,43 @@ def test_fast_path_maximum_recovery(dev, D, pattern, causal, density):
     close(o_fast, o_ref)
     close(o_exact, o_ref)
     close(o_fast, o_exact)
+
+
+@pytest.mark.parametrize("D,H,N", [(128, 8, 16384), (64, 16, 12352)])
+def test_paced_launch_is_bit_identical(dev, D, H, N, monkeypatch):
+    """PARO_ATTN_PACED (resident workgroups per XCD that take their q-blocks generation by generation)
+    against PARO_ATTN_UNPACED: the launch form may not change a single bit, whether the workgroups wait
+    for each other (default) or never do (a spin limit of zero, forced through the environment: the
+    meeting point only paces).  Shapes with more q-blocks per XCD than workgroups fit on it, so that the
+    paced kernel really runs several generations; checked against the oracle on one head."""
+    from paroatten_amd import _qattn_sm80 as qattn
+    from paroatten_amd import quant as Q
+    B = 1
+    nb = (N + 63) // 64
+    q, k, v = synth.make_qkv_device(B, H, N, D, torch.bfloat16, seed=5, device=dev)
+    mask = synth.make_block_mask(H, nb, 0.25, seed=6, device=dev)
+    mask[1, 7] = False     # an empty row in the middle of a generation
+    q8, qs, k8, ks = Q.per_warp_int8(q, k, None, BLKQ=64, WARPQ=32, BLKK=64)
+    v8, vsc, vm = Q.per_channel_fp8(v)
+    outs = []
+    for pacing, spins in ((False, None), (True, None), (True, "0"), (True, "3")):
+        if spins is None:
+            monkeypatch.delenv("PARO_ATTN_PACE_SPINS", raising=False)
+        else:
+            monkeypatch.setenv("PARO_ATTN_PACE_SPINS", spins)
+        out = torch.full_like(q, float("nan"))
+        lse = qattn.attn_sparse_prepacked(q8, k8, v8, vsc, vm, out, qs, ks, D ** -0.5, mask, return_lse=1, pacing=pacing)
+        outs.append((out, lse))
+    for o, l in outs[1:]:
+        assert torch.equal(o.view(torch.int16), outs[0][0].view(torch.int16)) and torch.equal(l, outs[0][1])
+    assert torch.count_nonzero(outs[0][0][0, 1, 7 * 64:8 * 64]) == 0
+    h = 3
+    o_ref, _ = O.sparse_attention(q8[:, h:h + 1].cpu(), k8[:, h:h + 1].cpu(), v[:, h:h + 1].cpu(), qs[:, h:h + 1].cpu(),
+                                  ks[:, h:h + 1].cpu(), mask[None, h:h + 1].cpu(), D ** -0.5, out_dtype=torch.float32)
+    _assert_close(outs[1][0][:, h:h + 1].cpu(), o_ref, baseline_shape=True)
+    # the fast-exponential instantiation and the folded inverse permutation go through the same launch code
+    a = torch.empty_like(q)
+    b = torch.empty_like(q)
+    qattn.attn_sparse_prepacked(q8, k8, v8, vsc, vm, a, qs, ks, D ** -0.5, mask, pacing=False)
+    qattn.attn_sparse_prepacked(q8, k8, v8, vsc, vm, b, qs, ks, D ** -0.5, mask, pacing=True)
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
