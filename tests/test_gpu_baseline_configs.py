@@ -194,3 +194,39 @@ def test_cfg4_wan720p_full_extent(dev, dtype):
             err = (got - ref).abs().max().item()
             assert err <= ATOL, (density, h, err)
             assert cosine(got, ref) >= COS, (density, h, cosine(got, ref))
+
+
+def test_cfg2_peaked_rows_fast_and_exact_exponential(dev, record_property):
+    """Peaked rows at the CogVideoX shape (RoPE turns the per-channel K bias into rows that one to three
+    keys dominate, outputs up to ~0.9 instead of ~0.05): what the default (fast) and the exact
+    exponential each deliver there.  Measured: both keep cosine >= 0.999 (fast 0.99921, exact 0.99935)
+    and both leave atol 2e-2 on a few 1e-5 of the elements (max |err| 0.05-0.09 on outputs of ~0.9: the
+    6 % worst-case relative rounding of an e4m3 V entry or P weight that a dominating key carries); the
+    fast path's share of that is the smaller one.  So on such rows neither path holds a FLAT atol 2e-2;
+    the bound that holds for both is the relative one of _fp8_bound_ok."""
+    import paroatten_amd as P
+    from paroatten_amd import permute as PM
+    from paroatten_amd import rope
+    wl = synth.WORKLOADS["cogvideox5b"]
+    H, N, D, nb = 2, wl.N, wl.D, wl.nb
+    q, k, v = synth.make_qkv(1, H, N, D, wl.dtype, seed=78)
+    mask = synth.make_block_mask(H, nb, 0.3, seed=79)
+    plan = synth.make_permute_plan(1, H, seed=80)
+    cos, sin = rope.rope_table_cog(D, wl.grid)
+    orders = PM.head_orders(plan, 0, dev)
+    qp, kp, vp = PM.rope_permute(q.to(dev), k.to(dev), v.to(dev), orders, wl.grid, wl.n_text, cos.to(dev), sin.to(dev))
+    ref = O.paro_path(q, k, v, mask[None], plan, 0, wl.grid, wl.n_text, cos, sin)
+    assert ref.float().abs().max().item() > 0.5       # the rows are peaked: i.i.d. inputs give ~0.05
+    res = {}
+    for name, exact in (("fast", False), ("exact", True)):
+        o = P.paroattn_qk_int8_pv_fp16_cuda(qp, kp, vp, mask.to(dev), smooth_k=True, exact_exp=exact)
+        o = PM.permute_inverse(o.contiguous(), orders, wl.grid, wl.n_text).cpu()
+        e = (o.float() - ref.float()).abs()
+        res[name] = (e.max().item(), (e > ATOL).float().mean().item(), cosine(o, ref))
+        record_property(f"{name}_max_abs_err", res[name][0])
+        record_property(f"{name}_frac_above_atol", res[name][1])
+        record_property(f"{name}_cosine", res[name][2])
+        assert res[name][2] >= COS, (name, res[name])
+        assert _fp8_bound_ok(o, ref), (name, res[name])
+        assert res[name][1] <= 2e-4, (name, res[name])          # atol 2e-2 holds on all but ~1e-5..1e-4 of the elements
+    assert res["exact"][2] >= res["fast"][2] - 1e-5              # the exact exponential is the (slightly) more accurate one
