@@ -346,12 +346,18 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   float d_exact = 0.f;  // LSE only: sum of the unrounded P~ of this lane's 32 kv-columns per block
 
   // ---- prologue ------------------------------------------------------------------------------
-  // K ring: stage j%3 holds the K tile of block j; V ring likewise.  Block i's S^T is produced one
-  // iteration ahead of its softmax and its P.V one iteration behind:
-  //   iteration i:  DMA K(i+3), V(i+1) | reads K(i+1), V(i-1) | S(i+1) = K(i+1).Q | P(i) = softmax(S(i))
-  //                 | O += V(i-1).P(i-1)
-  // What iteration i issues is waited for at the end of iteration i+1 (vmcnt keeps the newest
-  // LOADS_PER_IT in flight) and published by that iteration's barrier.
+  // K ring: stage j % NST holds the K tile of block j; V ring likewise.  One iteration per kept block, in
+  // two phases that never mix:
+  //   VALU phase   P~(i) = softmax weights of S(i) as e4m3 words (no matrix instruction in it)
+  //   matrix phase S(i+1) = K(i+1).Q, then O += V(i).P~(i) and the row sums, issued back to back
+  // A matrix instruction cannot be issued while the matrix pipe is busy, and a wave that meets one stalls
+  // in order; with the products sprinkled through the VALU stream every wave of a SIMD keeps running
+  // into the products of its neighbours and the VALU idles with them.  Kept apart, the VALU phase of one
+  // wave never blocks while the other waves of the SIMD take their turns on the matrix pipe, and the
+  // wave's own P.V products run under the VALU phase of its next block (which needs S(i+1) only).
+  //   D = 64  (three stages): iteration i requests K(i+3), V(i+2); what it requests is waited for at the
+  //                           end of iteration i+1 (vmcnt keeps the newest LOADS_PER_IT in flight)
+  //   D = 128 (two stages):   iteration i requests K(i+2), V(i+1) at its start and waits for them at its end
   int kb_c = __builtin_amdgcn_readfirstlane((int)klist[0]);
   int kb_1 = __builtin_amdgcn_readfirstlane((int)klist[1]);
   int kb_2 = __builtin_amdgcn_readfirstlane((int)klist[2]);
@@ -359,14 +365,10 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   constexpr bool RING2 = Lds::NST == 2;
   load_k(kb_c, 0);
   load_k(kb_1, 1);
-  if constexpr (RING2) {
-    // stage of block j: j % 2.  Iteration i: DMA K(i+2) and V(i) | reads K(i+1), V(i-1); everything an
-    // iteration requests has landed by the barrier at its end
-    load_v(kb_c, 1);  // the first iteration multiplies this stage by an all-zero P: it must hold finite values
-  } else {
-    load_v(kb_c, 0);
-    load_v(kb_c, 2);  // as above
+  load_v(kb_c, 0);
+  if constexpr (!RING2) {
     load_k(kb_2, 2);
+    load_v(kb_1, 1);
   }
   float c_cur = qsc * clist[0];
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -377,10 +379,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   // stage 0 is the first one the loop refills: both waves must hold their K(0) fragments by then
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
-  v8i pf_a = {0, 0, 0, 0, 0, 0, 0, 0}, pf_b = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // the pending product O^T += V8^T(prev) . P~^T(prev), plus the row sums of the ROUNDED P~ from one
-  // more MFMA against ones; idx 0..DT_TILES-1 = output tiles, DT_TILES = row sums
+  // the product O^T += V8^T . P~^T, plus the row sums of the ROUNDED P~ from one more MFMA against the
+  // selector operand; idx 0..DT_TILES-1 = output tiles, DT_TILES = row sums
   v4i vfrag[DT_TILES][2];
   auto pv_one = [&](const v8i& pf, int idx) {
     if (idx < DT_TILES) {
@@ -400,22 +401,18 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   };
 
   constexpr int N_PV = DT_TILES + 1;     // MFMAs of one P.V (+ row sums)
-  // One block.  `acc` holds its S^T on entry and that of the next block on exit: row tile 0 is
-  // consumed by chunks 0-3 of the stream below and re-issued right after them, row tile 1 after the
-  // last chunk.  `pf` receives the block's P~, `pf_p` holds that of the previous block.  sk1: K stage
-  // of block it+1; svp/sv1: V stages of blocks it-1 / it+1; K(it+3) goes to the stage K(it) has just
-  // left (sk0).
-  auto step = [&](int it, int sk0, int sk1, int svp, int sv1, v8i& pf, v8i& pf_p) {
+  // One block.  `acc` holds its S^T on entry and that of the next block on exit.  sk1: K stage of block
+  // it+1; sv: V stage of block it; skn / svn: the stages this iteration's DMA refills.
+  auto step = [&](int it, int sk1, int sv, int skn, int svn) {
     // -- memory traffic of this iteration, issued up front
     if constexpr (RING2) {
-      load_k(kb_2, sk0);   // K(it+2) into the stage K(it) has left
-      load_v(kb_c, sk0);   // V(it) into the stage V(it-2) has left
+      load_k(kb_2, skn);   // K(it+2) into the stage K(it) has left
+      load_v(kb_1, svn);   // V(it+1) into the stage V(it-1) has left
     } else {
-      load_k(kb_3, sk0);
-      load_v(kb_1, sv1);
+      load_k(kb_3, skn);   // K(it+3) into the stage K(it) has left
+      load_v(kb_2, svn);   // V(it+2) into the stage V(it-1) has left
     }
     const int kidx_v = (int)klist[it + 4];
-    read_v_frags(svp);
     const float c_next = qsc * clist[it + 1];
     // scale of this block and what follows from it and from the current maximum alone
     const float c = c_cur;
@@ -424,7 +421,6 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
     float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: byte = (8*(t + 7) + shift) / 32767
 
-    // -- row maximum of this block
     float s[2][16];
 #pragma unroll
     for (int mt = 0; mt < 2; mt++)
@@ -462,14 +458,12 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       smax = max3(smax, mx3, mx3);
       return fmaf(partner_max(smax), c, nmc);
     };
-    // Refresh of the running maximum: the new maximum applies to this block's weights at once; O and
-    // the row sums, which the pending P.V of the previous block still has to reach through the stream
-    // below, are rescaled after the stream.  Everything that depends on m only (threshold, offsets of
-    // the affine maps) is state that changes here.
-    float alpha = 1.0f;
+    // Refresh of the running maximum.  Everything that depends on m only (threshold, offsets of the
+    // affine maps) is state that changes here; O and the row sums hold every product up to the previous
+    // block by now and are rescaled on the spot.
     auto apply_refresh = [&](float m_blk) {
       const float m_new = fmaxf(m_i, m_blk);
-      alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+      const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
       m_i = m_new;
       m_thr = m_new + P_HEADROOM;
       m_off = P_EXP_OFFSET - m_new;
@@ -477,108 +471,78 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       bias = fmaf(-S_MAGIC_F, c, m_off);
       bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
       if constexpr (LSE) d_exact *= alpha;
+      d_acc[0] *= alpha;                                          // lanes 0..15: q-row lane
+      d_acc[1] *= __shfl(alpha, (lane & 15) + 16, 64);            // and q-row lane+16
+#pragma unroll
+      for (int dt = 0; dt < DT_TILES; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
     };
-    // Exact path: lazy refresh decided up front from the block maximum (P~ <= 2^(OFFSET + HEADROOM)).
-    // Fast path: optimistic, see below.
-    constexpr bool OPTIMISTIC = !EXACT;
-    bool refresh = false;
-    if constexpr (!OPTIMISTIC) {
-      const float m_blk = block_max();
-      refresh = __ballot(m_blk > m_thr) != 0ull;
-      if (refresh) apply_refresh(m_blk);
-    }
 
-    // -- the softmax weights of this block in 8 chunks (one 32-bit word of four e4m3 values each);
-    //    after each chunk one MFMA goes to the matrix pipe: first S^T of the NEXT block, then the
-    //    pending P.V of the PREVIOUS block.  All their operands are ready before the stream starts.
-    float rs = 0.f;
-    // MFMA issue plan: the pending P.V first (its operands are ready), S^T row tile 0 of the next
-    // block once chunk 3 has read the last of the current one, row tile 1 after chunk 7
-    // The K fragments of the next block (k-step r, both row tiles) are fetched from LDS right after
-    // the P.V MFMA that was the last reader of V fragment r: the two fragment sets never live at the
-    // same time and share registers.
-    auto mfma_after_chunk = [&](int r) {
-      if (r < DT_TILES) {
-        pv_one(pf_p, r);
-        read_k_frag(sk1, 2 * r);
-        read_k_frag(sk1, 2 * r + 1);
-      }
-      if (r == DT_TILES - 1 + (D == 64)) pv_one(pf_p, DT_TILES);   // row sums: chunk 2 (D = 64) / 3 (D = 128)
-      if constexpr (!OPTIMISTIC) {
-        if constexpr (D == 64) {
-          if (r == 3) qk_one(0);
-          else if (r == 4) qk_one(1);
-          else if (r == 7) { qk_one(2); qk_one(3); }
-        } else {
-          if (r == 4) { qk_one(0); qk_one(1); }
-          else if (r == 5) qk_one(2);
-          else if (r == 6) qk_one(3);
-          else if (r == 7) { qk_one(4); qk_one(5); qk_one(6); qk_one(7); }
-        }
-      }
-    };
-    // Fast path: the e4m3 byte of 2^t is built directly: byte = round(8*(t + 7) + FAST_EXP_SHIFT), i.e.
-    // exponent field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of
-    // two (at most 6 % off, shifted to be centred).  Per word of four weights: four fmas (the affine
-    // map pre-divided by 32767, result clamped to [0,1], which sends masked and underflowing elements to
-    // 0), two v_cvt_pknorm_i16_f32 (each rounds two values to 16-bit integer fields) and one shift-or
-    // that interleaves the two pairs into bytes.  Instead of fma + v_exp_f32 + half a packed FP8
-    // conversion per weight.  Chunk r = word r%4 of row tile r/4.
-    //
-    // It is optimistic about the maximum: the weights are computed with the running maximum as it
-    // is, and a packed 3-input maximum per chunk keeps the largest field seen.  A field above 126
-    // (the code of 448, the largest e4m3 value; fields cannot exceed 0x7FFF) means some score was more
-    // than 3.8 octaves above the running maximum: only then, and on the first block, is the block
-    // maximum searched (17 v_max3 otherwise spent on every block), the maximum refreshed and the
-    // eight words computed again.  For this the S^T MFMAs of the next block, which overwrite the
-    // scores, are all issued after the check.
-    auto fast_words = [&](auto&& after_chunk, int& ovf) {
-      float u_cur[4], u_nxt[4];
-#pragma unroll
-      for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], c8, bias8);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int r = 0; r < 8; r++) {
-        // the fmas of the next chunk are issued between this chunk's conversions: every conversion
-        // finds its input ready
-        const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
-        if (rn < 8) {
-          u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
-          u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8, bias8);
-        }
-        const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
-        __builtin_amdgcn_sched_barrier(0);
-        if (rn < 8) {
-          u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
-          u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8, bias8);
-        }
-        const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
-        __builtin_amdgcn_sched_barrier(0);
-        pf[r] = lshl8_or(hi, lo);
-        ovf = pk_max3_fields(ovf, lo, hi);
-#pragma unroll
-        for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
-        __builtin_amdgcn_sched_barrier(0);
-        after_chunk(r);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
+    // -- VALU phase: the softmax weights of this block as 8 words of four e4m3 values each
+    v8i pf;
+    constexpr bool OPTIMISTIC = !EXACT;
     if constexpr (OPTIMISTIC) {
+      // Fast path: the e4m3 byte of 2^t is built directly: byte = round(8*(t + 7) + FAST_EXP_SHIFT), i.e.
+      // exponent field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of
+      // two (at most 6 % off, shifted to be centred).  Per word of four weights: four fmas (the affine
+      // map pre-divided by 32767, result clamped to [0,1], which sends masked and underflowing elements to
+      // 0), two v_cvt_pknorm_i16_f32 (each rounds two values to 16-bit integer fields) and one shift-or
+      // that interleaves the two pairs into bytes.  Instead of fma + v_exp_f32 + half a packed FP8
+      // conversion per weight.  Word r = word r%4 of row tile r/4.
+      //
+      // It is optimistic about the maximum: the weights are computed with the running maximum as it
+      // is, and a packed 3-input maximum per word keeps the largest field seen.  A field above 126
+      // (the code of 448, the largest e4m3 value; fields cannot exceed 0x7FFF) means some score was more
+      // than 3.8 octaves above the running maximum: only then, and on the first block, is the block
+      // maximum searched (17 v_max3 otherwise spent on every block), the maximum refreshed and the
+      // eight words computed again (the scores are still in `acc`: the next block's S^T is issued below).
+      auto fast_words = [&](int& ovf) {
+        float u_cur[4], u_nxt[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], c8, bias8);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+          // the fmas of the next word are issued between this word's conversions: every conversion
+          // finds its input ready
+          const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
+          if (rn < 8) {
+            u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
+            u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8, bias8);
+          }
+          const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (rn < 8) {
+            u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
+            u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8, bias8);
+          }
+          const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
+          __builtin_amdgcn_sched_barrier(0);
+          pf[r] = lshl8_or(hi, lo);
+          ovf = pk_max3_fields(ovf, lo, hi);
+#pragma unroll
+          for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      };
       int ovf = 0;
-      fast_words(mfma_after_chunk, ovf);
+      fast_words(ovf);
       const unsigned top = max((unsigned)ovf & 0xffffu, (unsigned)ovf >> 16);
-      refresh = it == 0 || __ballot(top > 126u) != 0ull;
-      if (refresh) {
+      if (it == 0 || __ballot(top > 126u) != 0ull) {
         apply_refresh(block_max());
         int ovf2 = 0;
-        fast_words([](int) {}, ovf2);
+        fast_words(ovf2);
       }
-      qk_mfma();
     } else {
+      // Exact path: lazy refresh decided up front from the block maximum (P~ <= 2^(OFFSET + HEADROOM)),
+      // then P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential and the packed FP8 conversion
+      const float m_blk = block_max();
+      if (__ballot(m_blk > m_thr) != 0ull) apply_refresh(m_blk);
+      float rs = 0.f;
 #pragma unroll
       for (int r = 0; r < 8; r++) {
         const int mt = r >> 2, i0 = 4 * (r & 3);
-        // P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential, then the packed FP8 conversion
         const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
         const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
         const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
@@ -588,24 +552,29 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
         cvt_pk_fp8<false>(w, p0, p1);
         cvt_pk_fp8<true>(w, p2, p3);
         pf[r] = w;
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_after_chunk(r);
-        __builtin_amdgcn_sched_barrier(0);
       }
+      if constexpr (LSE) d_exact += rs;
     }
-    if constexpr (LSE) d_exact += rs;
-    if (it + 1 < cnt) dump_s(kb_1);
-    if (refresh) {
-      d_acc[0] *= alpha;                                          // lanes 0..15: q-row lane
-      d_acc[1] *= __shfl(alpha, (lane & 15) + 16, 64);            // and q-row lane+16
-#pragma unroll
-      for (int dt = 0; dt < DT_TILES; dt++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) o_acc[dt][i] *= alpha;
-    }
+    __builtin_amdgcn_sched_barrier(0);
 
-    // -- everything the PREVIOUS iteration sent to LDS has to have landed before the barrier
-    //    publishes it; this iteration's own DMA may stay in flight
+    // -- matrix phase: S^T of the next block first (the next VALU phase waits for it alone), then this
+    //    block's P.V and row sums, which run on under that VALU phase
+    read_k_frags(sk1);
+    if constexpr (D == 64) read_v_frags(sv);
+    __builtin_amdgcn_sched_barrier(0);
+    qk_mfma();
+    __builtin_amdgcn_sched_barrier(0);
+    // (D = 128: the V fragments go into the registers the K fragments have just left)
+    if constexpr (D == 128) {
+      read_v_frags(sv);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int i = 0; i < N_PV; i++) pv_one(pf, i);
+    __builtin_amdgcn_sched_barrier(0);
+    if (it + 1 < cnt) dump_s(kb_1);
+
+    // -- what the ring needs next has to have landed before the barrier publishes it
     const int kb_4 = __builtin_amdgcn_readfirstlane(kidx_v);
     // (a bare s_barrier: __syncthreads() would add a fence that waits for ALL outstanding loads)
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(RING2 ? 0 : LOADS_PER_IT) : "memory");
@@ -615,36 +584,26 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   };
 
   if constexpr (RING2) {
-    // stage of block j is j % 2: the step refills stage it % 2 and reads K(it+1), V(it-1) from the other
+    // stage of block j is j % 2: iteration `it` reads K(it+1) from the other stage and V(it) from its own,
+    // refills its own K stage with K(it+2) and the other V stage with V(it+1)
     for (int it = 0; it < cnt; it += 2) {
-      step(it, 0, 1, 1, 0, pf_a, pf_b);
+      step(it, 1, 0, 0, 1);
       if (it + 1 >= cnt) break;
-      step(it + 1, 1, 0, 0, 1, pf_b, pf_a);
+      step(it + 1, 0, 1, 1, 0);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    // the last block's P.V is still pending; its V tile sits in stage (cnt-1) % 2
-    read_v_frags((cnt - 1) & 1);
-    const v8i& pf_last = (cnt & 1) ? pf_a : pf_b;
-#pragma unroll
-    for (int i = 0; i < N_PV; i++) pv_one(pf_last, i);
   } else {
-    // stage of block j is j % 3: with i = it % 3 the step writes K stage i, reads K stage i+1, reads V
-    // stage i-1 and writes V stage i+1
-    int i3 = 0;  // it % 3
-    for (int it = 0; it < cnt; it += 2) {
-      const int s1 = i3 == 2 ? 0 : i3 + 1, s2 = 3 - i3 - s1;  // (i3+1)%3 and the remaining stage (i3+2)%3
-      step(it, i3, s1, s2, s1, pf_a, pf_b);
-      if (it + 1 >= cnt) { i3 = s1; break; }
-      step(it + 1, s1, s2, i3, s2, pf_b, pf_a);
-      i3 = s2;
+    // stage of block j is j % 3: with i = it % 3, iteration `it` reads K stage i+1 and V stage i, refills
+    // K stage i with K(it+3) and V stage i+2 with V(it+2)
+    // (unrolled by three: the stage numbers are constants and every LDS address an immediate offset)
+    for (int it = 0; it < cnt; it += 3) {
+      step(it, 1, 0, 0, 2);
+      if (it + 1 >= cnt) break;
+      step(it + 1, 2, 1, 1, 0);
+      if (it + 2 >= cnt) break;
+      step(it + 2, 0, 2, 2, 1);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // DMA of the padded tail blocks: nobody reads it
-    // the last block's P.V is still pending: i3 is now cnt % 3, its V tile sits in stage (cnt-1) % 3
-    read_v_frags(i3 == 0 ? 2 : i3 - 1);
-    const v8i& pf_last = (cnt & 1) ? pf_a : pf_b;
-#pragma unroll
-    for (int i = 0; i < N_PV; i++) pv_one(pf_last, i);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // DMA of the padded tail blocks: nobody reads it
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------
   const float d_lo = __shfl(d_acc[0], l32 & 15, 64), d_hi = __shfl(d_acc[1], l32 & 15, 64);
