@@ -79,6 +79,28 @@ def event_time_ms(fn, reps, warmup):
     return e0.elapsed_time(e1) / reps
 
 
+def mfma_ceiling(lib, L, dev):
+    """Sustained rate of back-to-back MFMAs alone (no memory traffic, no VALU work), 4 waves per SIMD."""
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = torch.randint(-2 ** 31, 2 ** 31 - 1, (64 * 16,), generator=g, device=dev, dtype=torch.int64).to(torch.int32)
+    # e4m3 bytes without NaN codes (0x7f / 0xff), so that the fp8 products stay finite
+    b = rnd.view(torch.uint8)
+    b[(b & 0x7F) == 0x7F] = 0x3C
+    zero = torch.zeros_like(rnd)
+    wgs, iters = 256 * 4, 20000
+    sink = torch.empty(wgs * 4, dtype=torch.float32, device=dev)
+    out = {"metric": "sustained MFMA rate, back-to-back instructions only", "unit": "TOP/s",
+           "peak_nominal": PEAK_MFMA_TOPS, "workgroups": wgs, "iters": iters}
+    for kind, kname in ((0, "int8_32x32x32"), (1, "fp8_32x32x64")):
+        ops = lib.paro_diag_mfma_loop_ops(kind, wgs, iters)
+        for oname, buf in (("random", rnd), ("zero", zero)):
+            fn = lambda: L.check(lib.paro_diag_mfma_loop(kind, L.ptr(buf), L.ptr(sink), wgs, iters, L.stream_of(sink)))
+            t = event_time_ms(fn, 10, 2)
+            out[f"{kname}_{oname}"] = {"ms": round(t, 3), "tops": round(ops / (t * 1e-3) / 1e12, 1),
+                                       "frac_nominal": round(ops / (t * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 3)}
+    return out
+
+
 def cpu_model_name():
     try:
         with open("/proc/cpuinfo") as f:
@@ -156,6 +178,9 @@ def main():
     ap.add_argument("--pacing", choices=["auto", "on", "off"], default="auto",
                     help="attention launch: generation-paced resident workgroups (on), the plain launch (off), or the "
                          "library's own choice (auto: paced when one head's K8+V8 exceed an XCD's L2)")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="only time back-to-back MFMAs (int8 and fp8, random and zero operands): what the matrix pipe "
+                         "sustains on this box, the ceiling of any kernel built on it.  Prints its own JSON line.")
     ap.add_argument("--exact-exp", action="store_true", help="attention kernel with exact exponentials (flag PARO_ATTN_EXACT_EXP)")
     args = ap.parse_args()
     if args.pacing != "auto":   # the library's default for calls that carry neither pacing flag
@@ -177,6 +202,9 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     lib = L.load()
+    if args.mfma_ceiling:
+        print(json.dumps(mfma_ceiling(lib, L, dev)))
+        return
     wl = synth.WORKLOADS[args.workload]
     global HEADLINE_DENSITY, DENSITIES
     HEADLINE_DENSITY, DENSITIES = WORKLOAD_DENSITIES[args.workload]

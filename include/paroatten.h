@@ -309,6 +309,17 @@ int64_t paro_mask_bits_bytes(int64_t n);
 int paro_mask_pack(const uint8_t* mask, uint8_t* bits, int64_t n, void* stream);
 int paro_mask_unpack(const uint8_t* bits, uint8_t* mask, int64_t n, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Measurement aid (no counterpart in the reference): `workgroups` workgroups of four waves each issue
+ * `iters` x 4 back-to-back MFMAs of the kind the attention kernel uses (kind 0: v_mfma_i32_32x32x32_i8,
+ * kind 1: v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands) with nothing else in the loop.  operands: 4 KiB of
+ * device memory (64 lanes x 16 words) that every wave takes its A / B registers from (random bytes or
+ * zeros); sink: one float per wave (workgroups * 4).  paro_diag_mfma_loop_ops() = operations one launch
+ * executes.  Timed by the caller, it gives what the matrix pipe sustains on the GPU at hand.
+ * ------------------------------------------------------------------------------------------- */
+int64_t paro_diag_mfma_loop_ops(int kind, int workgroups, int iters);
+int paro_diag_mfma_loop(int kind, const void* operands, float* sink, int workgroups, int iters, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

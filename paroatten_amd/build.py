@@ -22,7 +22,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIBDIR = PKG / "lib"
 LIB = LIBDIR / "libparoatten_hip.so"
-SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "v_channel.hip", "rope_permute.hip", "fused_prep.hip", "mask_bits.hip", "attn_sparse.hip"]
+SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "v_channel.hip", "rope_permute.hip", "fused_prep.hip", "mask_bits.hip", "diag.hip", "attn_sparse.hip"]
 ARCH = "gfx950"
 
 FLAGS = [
