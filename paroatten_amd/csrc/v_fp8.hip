@@ -174,24 +174,29 @@ __global__ void __launch_bounds__(256) v_pack_kernel(const unsigned short* __res
   }
 }
 
-// v_mean += v_scale * (sum over tiles and row tiles of the residual sums) / N; 1024 / D slices of the
-// tile range per channel, combined through LDS in a fixed order
+// v_mean += v_scale * (sum over tiles and row tiles of the residual sums) / N.  A thread takes four
+// channels of every SL-th row (16-byte loads, all independent), the SL partial sums per channel are
+// combined through LDS in a fixed order.
 template <int D>
 __global__ void __launch_bounds__(1024) v_residual_kernel(const float* __restrict__ resid,
                                                           const float* __restrict__ v_scale,
                                                           float* __restrict__ v_mean, int N, int n_rows) {
-  constexpr int SL = 1024 / D;
-  __shared__ float red[SL][D];
-  const int ch = threadIdx.x % D, sl = threadIdx.x / D;
+  constexpr int C4 = D / 4;          // threads per row
+  constexpr int SL = 1024 / C4;      // rows in flight per pass
+  __shared__ v4f red[SL][C4];
+  const int c4 = threadIdx.x % C4, sl = threadIdx.x / C4;
   const int64_t bh = blockIdx.x;
-  const float* p = resid + bh * n_rows * D;
-  float s = 0.f;
-  for (int c = sl; c < n_rows; c += SL) s += p[(int64_t)c * D + ch];
-  red[sl][ch] = s;
+  const v4f* p = reinterpret_cast<const v4f*>(resid + bh * n_rows * D) + c4;
+  v4f s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int r = sl; r < n_rows; r += SL) s += p[(int64_t)r * C4];
+  red[sl][c4] = s;
   __syncthreads();
-  if (sl == 0) {
-    for (int i = 1; i < SL; i++) s += red[i][ch];
-    v_mean[bh * D + ch] += v_scale[bh * D + ch] * (s / (float)N);
+  if (threadIdx.x < D) {
+    const int ch = threadIdx.x;
+    float t = 0.f;
+    for (int i = 0; i < SL; i++) t += red[i][ch >> 2][ch & 3];
+    v_mean[bh * D + ch] += v_scale[bh * D + ch] * (t / (float)N);
   }
 }
 
