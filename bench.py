@@ -45,10 +45,16 @@ WORKLOAD_DENSITIES = {
     "wan14b_480p": (0.3, (0.3,)),
     "wan14b_720p": (0.2, (0.2, 1.0)),     # 1.0 = the dense comparison run
 }
-# HBM bytes per attention-kernel launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/path_kernels_cogvideox5b_hbm_traffic.txt): FETCH_SIZE 166963 x 2.0 KiB + WRITE_SIZE 213836 x 1.0 KiB,
-# the factors being what the same counters read for a plain copy of known size; the same at every density
-ATTN_TRAFFIC_BYTES = int((166963 * 2.0 + 213836 * 1.0) * 1024)
+# HBM-side bytes per attention-kernel launch at the headline density, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/attn_sparse_hbm_traffic_by_workload.txt): counter mean per dispatch x 2.0 KiB (FETCH_SIZE) or
+# x 1.0 KiB (WRITE_SIZE), the factors being what the same counters read for a plain copy of known size.
+# CogVideoX: the same at every density (one head's K8 + V8 stay in the L2).  Wan: L2 fills, with the paced
+# launch; they vary by tens of percent from box to box at 720p, where a head is five times the L2.
+ATTN_TRAFFIC_BYTES = {
+    "cogvideox5b": int((167468 * 2.0 + 213796 * 1.0) * 1024),
+    "wan14b_480p": int((744582 * 2.0 + 328686 * 1.0) * 1024),
+    "wan14b_720p": int((12405556 * 2.0 + 771465 * 1.0) * 1024),
+}
 
 
 SETTLE_MS = 60.0   # load the chip this long before a measurement: after any pause the shader clock
@@ -299,7 +305,7 @@ def main():
         "peak": PEAK_MFMA_TOPS,
         "unit": "TOP/s",
         "frac": round(achieved / PEAK_MFMA_TOPS, 4),
-        "traffic": ATTN_TRAFFIC_BYTES if args.workload == "cogvideox5b" else None,
+        "traffic": ATTN_TRAFFIC_BYTES.get(args.workload) if args.pacing == "auto" and not args.zero_operands else None,
         "ops_per_launch": hk["kept_blocks"] * 4.0 * 64 * 64 * D,
         "avg_launch_ms": hk["attn_kernel_ms"],
     }
