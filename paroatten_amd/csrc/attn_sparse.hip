@@ -133,7 +133,11 @@ template <int D> struct AttnLds {
   static constexpr int KTILE = 64 * D;   // bytes of one K8 tile: 64 rows of D bytes, 16-byte chunks XOR-swizzled
   static constexpr int VTILE = 64 * D;   // bytes of one V8 tile (fragment order, as in HBM)
   static constexpr int V_OFF = NST * KTILE;
-  static constexpr int LIST_OFF = NST * (KTILE + VTILE);
+  static constexpr int EPI_OFF = NST * (KTILE + VTILE);
+  // D = 64: v_scale and v_mean of the head (2 x D floats), fetched at the start so that the epilogue does not
+  // wait for them.  (At D = 128 the 1 KB would cost Wan 720p its fourth workgroup per CU.)
+  static constexpr int EPI_BYTES = D == 64 ? 2 * D * 4 : 0;
+  static constexpr int LIST_OFF = EPI_OFF + EPI_BYTES;
   static constexpr int LIST_PAD = 8;     // list entries past the end that the prefetch may touch
   // chunk c of row `row` is stored at chunk position c ^ swz(row): makes the MFMA A-operand reads (32
   // rows x one 16-byte chunk per half-wave) conflict-free; measured on gfx950 for both row lengths
@@ -164,9 +168,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   constexpr int CPR = D / 16;       // 16-byte chunks per K row
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  float* clist = reinterpret_cast<float*>(smem + Lds::LIST_OFF);  // [nbk + LIST_PAD] k_scale of kept blocks
-  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + p.nbk + Lds::LIST_PAD);  // their indices
-  __shared__ int s_cnt;
+  float* clist = reinterpret_cast<float*>(smem + Lds::LIST_OFF);  // [nbk + LIST_PAD + 1] k_scale of kept blocks
+  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + p.nbk + Lds::LIST_PAD + 1);  // their indices
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
@@ -177,39 +180,42 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   const int hk = h / (p.H / p.Hkv);
   const int64_t bhk = (int64_t)b * p.Hkv + hk;
 
-  // ---- compact list of kept k-blocks (and of their k scales) ------------------------------
+  // Everything the q-block needs from memory before its first tile is requested here in one go, without a
+  // branch (Q, the mask row, the k scales, the epilogue constants, the permutation order as a scalar): a
+  // workgroup lives for a few dozen block iterations only, and every dependent round trip to HBM in front
+  // of or behind its loop costs two or three of them.  Loads behind a branch are waited for one by one, and
+  // loads whose only use sits in a branch are moved into it; so both waves build the (identical) lists, and
+  // entries that are not kept go to a spare slot instead of being skipped.
+  const int order_h = p.orders != nullptr ? p.orders[h] : 0;
   const float* ksc_base = p.k_scale + bhk * p.nbk;
   const int kmax = CAUSAL ? min(p.nbk, qb + 1) : p.nbk;
-  if (wave == 0) {
-    const uint8_t* mrow = p.sparse + b * p.sparse_bs + ((int64_t)h * p.nbq + qb) * p.nbk;
-    int cnt = 0, last = 0;
-    for (int base = 0; base < kmax; base += 256) {
-      uint8_t m[4];
+  const uint8_t* mrow = p.sparse + b * p.sparse_bs + ((int64_t)h * p.nbq + qb) * p.nbk;
+  constexpr int MU = 8;   // 64 x MU blocks per pass: one pass up to 512 blocks
+  uint8_t m[MU];
+  float msc[MU];
+  auto list_load = [&](int base) {
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        const int j = base + u * 64 + lane;
-        m[u] = (j < kmax) ? mrow[j] : (uint8_t)0;
-      }
+    for (int u = 0; u < MU; u++) {
+      const int j = min(base + u * 64 + lane, kmax - 1);   // past the end: the last entry again
+      m[u] = mrow[j];
+      msc[u] = ksc_base[j];
+    }
+  };
+  const int trash = p.nbk + Lds::LIST_PAD;   // the spare slot
+  int cnt = 0;
+  auto list_take = [&](int base) {
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        const bool keep = m[u] != 0;
-        const unsigned long long bal = __ballot(keep);
-        if (keep) {
-          const int pos = cnt + __popcll(bal & ((1ull << lane) - 1ull));
-          klist[pos] = (unsigned short)(base + u * 64 + lane);
-          clist[pos] = ksc_base[base + u * 64 + lane];
-        }
-        cnt += __popcll(bal);
-        if (bal) last = base + u * 64 + 63 - __clzll(bal);
-      }
+    for (int u = 0; u < MU; u++) {
+      const int j = base + u * 64 + lane;
+      const bool keep = m[u] != 0 && j < kmax;
+      const unsigned long long bal = __ballot(keep);
+      const int pos = keep ? cnt + __popcll(bal & ((1ull << lane) - 1ull)) : trash;
+      klist[pos] = (unsigned short)j;
+      clist[pos] = msc[u];
+      cnt += __popcll(bal);
     }
-    // the loop prefetches up to 4 blocks ahead without branching: pad with the last kept block
-    if (lane < Lds::LIST_PAD) {
-      klist[cnt + lane] = (unsigned short)last;
-      clist[cnt + lane] = ksc_base[last];
-    }
-    if (lane == 0) s_cnt = cnt;
-  }
+  };
+  list_load(0);
 
   // ---- Q fragments (B operand: column = q-row, 16 channels per lane and k-step) -----------
   const int qrow = qb * 64 + wave * 32 + l32;
@@ -222,15 +228,39 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   }
   const float qsc = p.q_scale[((int64_t)b * p.H + h) * (p.nbq * 2) + qb * 2 + wave] * p.sm_scale_log2e;
 
+  float* epi = reinterpret_cast<float*>(smem + Lds::EPI_OFF);   // [2][D]: v_scale, v_mean (D = 64)
+  float epi_sc = 0.f, epi_mn = 0.f;
+  if constexpr (Lds::EPI_BYTES != 0) {
+    epi_sc = p.v_scale[bhk * D + lane];
+    if (p.v_mean) epi_mn = p.v_mean[bhk * D + lane];
+  }
+
+  // ---- compact list of kept k-blocks (and of their k scales) ------------------------------
+  list_take(0);
+  for (int base = 64 * MU; base < kmax; base += 64 * MU) {
+    list_load(base);
+    list_take(base);
+  }
+  // the loop prefetches up to 4 blocks ahead without branching: pad with the last kept block (entry
+  // cnt - 1 of the lists just written; LDS operations of one wave complete in order)
+  if (cnt > 0 && lane < Lds::LIST_PAD) {
+    klist[cnt + lane] = klist[cnt - 1];
+    clist[cnt + lane] = clist[cnt - 1];
+  }
+  if constexpr (Lds::EPI_BYTES != 0) {
+    epi[lane] = epi_sc;
+    epi[D + lane] = epi_mn;
+  }
+
   __syncthreads();
-  const int cnt = s_cnt;
+
 
   using OutT = F16x<OUT_DT>;
   // where this lane's q-row goes (evaluated where it is needed: nothing of it lives across the loop)
   auto out_row_ptr = [&]() {
     int drow = qrow;
     if (p.orders != nullptr && qrow >= p.n_text && qrow < p.Nq)
-      drow = p.n_text + unpermute_index(qrow - p.n_text, p.orders[h], p.F, p.Hh, p.W);
+      drow = p.n_text + unpermute_index(qrow - p.n_text, order_h, p.F, p.Hh, p.W);
     return reinterpret_cast<unsigned short*>(p.out) + b * p.os_b + h * p.os_h + (int64_t)drow * p.os_n;
   };
 
@@ -617,9 +647,14 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
 #pragma unroll
       for (int g = 0; g < 4; g++) {
         const int ch = 32 * dt + 8 * g + 4 * lh;
-        const v4f sc = *reinterpret_cast<const v4f*>(vsc + ch);
-        v4f mn = {0.f, 0.f, 0.f, 0.f};
-        if (vmn) mn = *reinterpret_cast<const v4f*>(vmn + ch);
+        v4f sc, mn = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (Lds::EPI_BYTES != 0) {
+          sc = *reinterpret_cast<const v4f*>(epi + ch);
+          mn = *reinterpret_cast<const v4f*>(epi + D + ch);
+        } else {
+          sc = *reinterpret_cast<const v4f*>(vsc + ch);
+          if (vmn) mn = *reinterpret_cast<const v4f*>(vmn + ch);
+        }
         unsigned short r[4];
 #pragma unroll
         for (int q = 0; q < 4; q++) r[q] = OutT::from_f32(fmaf(o_acc[dt][4 * g + q] * inv, sc[q], mn[q]));
@@ -717,7 +752,7 @@ static bool want_pacing(const AttnParams& p, int D) {
 
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
-  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + AttnLds<D>::LIST_PAD) * 6 + 15) & ~(size_t)15);
+  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + AttnLds<D>::LIST_PAD + 1) * 6 + 15) & ~(size_t)15);
   if (!DUMP && want_pacing(p, D)) {
     auto kern = attn_sparse_paced_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
     if (smem > 48 * 1024)
