@@ -149,10 +149,13 @@ template <int D> struct AttnLds {
 
 // LDS-DMA: 16 bytes per lane from a buffer straight into LDS at lds_base + lane*16; no registers, no
 // ds_write; completion is counted by vmcnt
+// IMM (a compile-time constant below 4096) is added to BOTH the memory offset and the LDS address: the
+// pieces of one tile share one LDS base register (M0) and differ in IMM only
+template <int IMM>
 __device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_base, int voffset,
                                                   int soffset) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_base, 16, voffset,
-                                           soffset, 0, 0);
+                                           soffset, IMM, 0);
 }
 
 // Waves per SIMD the register budget is set for: the D = 64 production variants fit 168 registers.
@@ -287,20 +290,28 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   for (int i = 0; i < NLD; i++) {
     const int pos = (wave_u * NLD + i) * 1024 + lane * 16;  // byte position inside the LDS tile
     const int row = pos / D, cpos = (pos % D) / 16;
-    k_goff[i] = row * (int)p.ks_n + ((cpos ^ Lds::swz(row)) * 16);
-    v_goff[i] = pos;
+    // (less the immediate offset i * 1024 that the instruction adds on both sides; row * ks_n >= i * 1024)
+    k_goff[i] = row * (int)p.ks_n + ((cpos ^ Lds::swz(row)) * 16) - i * 1024;
+    v_goff[i] = pos - i * 1024;
   }
   const int k_blk_stride = 64 * (int)p.ks_n;
   auto load_k = [&](int kb, int ST) {  // rows >= Nk read as 0
-#pragma unroll
-    for (int i = 0; i < NLD; i++)
-      buffer_load16_lds(k_rsrc, smem + ST * Lds::KTILE + (wave_u * NLD + i) * 1024, k_goff[i], kb * k_blk_stride);
+    uint8_t* base = smem + ST * Lds::KTILE + wave_u * NLD * 1024;
+    buffer_load16_lds<0>(k_rsrc, base, k_goff[0], kb * k_blk_stride);
+    buffer_load16_lds<1024>(k_rsrc, base, k_goff[1], kb * k_blk_stride);
+    if constexpr (NLD == 4) {
+      buffer_load16_lds<2048>(k_rsrc, base, k_goff[2], kb * k_blk_stride);
+      buffer_load16_lds<3072>(k_rsrc, base, k_goff[3], kb * k_blk_stride);
+    }
   };
   auto load_v = [&](int kb, int ST) {
-#pragma unroll
-    for (int i = 0; i < NLD; i++)
-      buffer_load16_lds(v_rsrc, smem + Lds::V_OFF + ST * Lds::VTILE + (wave_u * NLD + i) * 1024, v_goff[i],
-                        kb * Lds::VTILE);
+    uint8_t* base = smem + Lds::V_OFF + ST * Lds::VTILE + wave_u * NLD * 1024;
+    buffer_load16_lds<0>(v_rsrc, base, v_goff[0], kb * Lds::VTILE);
+    buffer_load16_lds<1024>(v_rsrc, base, v_goff[1], kb * Lds::VTILE);
+    if constexpr (NLD == 4) {
+      buffer_load16_lds<2048>(v_rsrc, base, v_goff[2], kb * Lds::VTILE);
+      buffer_load16_lds<3072>(v_rsrc, base, v_goff[3], kb * Lds::VTILE);
+    }
   };
   constexpr int LOADS_PER_IT = 2 * NLD;  // DMA instructions one wave issues per block
 
@@ -334,8 +345,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   v16i acc[2];
   // the MFMAs are issued one at a time from inside the VALU stream (see step below): a wave that
   // issues them back to back sits blocked behind the matrix pipe for their whole duration
-  auto qk_one = [&](int idx) {  // idx = mt * KS + ks, ks ascending per mt
-    const int mt = idx / KS, ks = idx % KS;
+  auto qk_one = [&](int idx) {
+    const int mt = idx / KS, ks = idx % KS;  // idx = mt * KS + ks, ks ascending per mt (alternating the row
+                                             // tiles instead measured the same)
     if (ks == 0) acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[mt], qf[0], magic, 0, 0, 0);
     else acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[ks * 2 + mt], qf[ks], acc[mt], 0, 0, 0);
   };
@@ -459,13 +471,20 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     // columns past the end of K (last block) or above the diagonal (causal) leave the softmax
     const bool edge = (kb_c == p.nbk - 1 && (p.Nk & 63) != 0) || (CAUSAL && kb_c == qb);
     if (edge) {
+      // One threshold per lane: the element of row tile mt, register i is column
+      // kb*64 + 4*lh + cidx, cidx = 32*mt + 8*(i/4) + i%4, and it is dead from the first column past the end
+      // of K (or above the diagonal) on.  (The block index is made opaque: from loop invariants the compiler
+      // would evaluate the 32 lane masks in front of the loop and hold them in 64 scalar registers.)
+      int kb_e = kb_c;
+      asm volatile("" : "+s"(kb_e));
+      int thr = p.Nk - kb_e * 64 - 4 * lh;
+      if constexpr (CAUSAL) thr = min(thr, qrow + 1 - kb_e * 64 - 4 * lh);
 #pragma unroll
       for (int mt = 0; mt < 2; mt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-          const int j = kb_c * 64 + 32 * mt + 8 * (i >> 2) + 4 * lh + (i & 3);
-          const bool dead = (j >= p.Nk) || (CAUSAL && j > qrow);
-          if (dead) s[mt][i] = -INFINITY;
+          const int cidx = 32 * mt + 8 * (i >> 2) + (i & 3);
+          if (cidx >= thr) s[mt][i] = -INFINITY;
         }
     }
 
