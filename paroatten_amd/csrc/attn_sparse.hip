@@ -93,9 +93,9 @@ __device__ __forceinline__ float fma_clamp01(float a, float b, float c) {
 
 // two floats in [0,1] -> round(x * 32767) as two 16-bit fields (never negative, at most 0x7FFF)
 __device__ __forceinline__ int cvt_pknorm_i16(float a, float b) {
-  int w;
-  asm("v_cvt_pknorm_i16_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));
-  return w;
+  // (the builtin, not inline assembly: between two assembly statements the compiler assumes the worst
+  // hazard and pads with s_nop)
+  return __builtin_bit_cast(int, __builtin_amdgcn_cvt_pknorm_i16(a, b));
 }
 
 // field-wise maximum of three words of two non-negative 16-bit integers each: on such bit patterns
@@ -105,12 +105,6 @@ __device__ __forceinline__ int pk_max3_fields(int a, int b, int c) {
   int r;
   asm("v_pk_maximum3_f16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
-}
-
-__device__ __forceinline__ int lshl8_or(int hi, int lo) {
-  int w;
-  asm("v_lshl_or_b32 %0, %1, 8, %2" : "=v"(w) : "v"(hi), "v"(lo));
-  return w;
 }
 
 __device__ __forceinline__ float partner_max(float x) {
@@ -340,8 +334,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   v16i magic;
 #pragma unroll
   for (int i = 0; i < 16; i++) magic[i] = S_MAGIC_BITS;
-  // D = 64 has registers to spare: keep the constant block resident instead of rebuilding it per block
-  if constexpr (D == 64) asm volatile("" : "+v"(magic));
+  // keep the constant block resident instead of rebuilding it per block (15 scalar + 8 vector moves)
+  // (not in the D = 128 variants with exact exponentials, which have no 16 registers to spare)
+  if constexpr (D == 64 || (!EXACT && !LSE && !DUMP)) asm volatile("" : "+v"(magic));
   v16i acc[2];
   // the MFMAs are issued one at a time from inside the VALU stream (see step below): a wave that
   // issues them back to back sits blocked behind the matrix pipe for their whole duration
@@ -552,22 +547,23 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
-          // the fmas of the next word are issued between this word's conversions: every conversion
-          // finds its input ready
+          // the fmas of the next word are issued behind this word's conversions: every conversion finds
+          // its input ready, and the shift-or is not the instruction right behind the conversion it reads
+          // (a packed 16-bit result needs one wait state before a full-register read)
           const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
+          const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
           if (rn < 8) {
             u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
             u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8, bias8);
           }
-          const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
           __builtin_amdgcn_sched_barrier(0);
+          const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
           if (rn < 8) {
             u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
             u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8, bias8);
           }
-          const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
           __builtin_amdgcn_sched_barrier(0);
-          pf[r] = lshl8_or(hi, lo);
+          pf[r] = (hi << 8) | lo;   // v_lshl_or_b32: the fields of hi move into the odd bytes
           ovf = pk_max3_fields(ovf, lo, hi);
 #pragma unroll
           for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
