@@ -188,6 +188,10 @@ def main():
                     help="only time back-to-back MFMAs (int8 and fp8, random and zero operands): what the matrix pipe "
                          "sustains on this box, the ceiling of any kernel built on it.  Prints its own JSON line.")
     ap.add_argument("--exact-exp", action="store_true", help="attention kernel with exact exponentials (flag PARO_ATTN_EXACT_EXP)")
+    ap.add_argument("--blocks-per-row", default=None, metavar="LIST",
+                    help="measurement aid: instead of the benchmark, time the attention kernel with masks that keep "
+                         "exactly n blocks in every row, for every n of the comma-separated list (0,1,2,4,...): what a "
+                         "q-block costs beyond its blocks")
     args = ap.parse_args()
     if args.pacing != "auto":   # the library's default for calls that carry neither pacing flag
         os.environ["PARO_ATTN_PACING"] = "1" if args.pacing == "on" else "0"
@@ -251,6 +255,18 @@ def main():
             L.ptr(out), L.DTYPE_CODE[out.dtype], None, None, B, H, H, N, N, D,
             q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
             out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, attn_flags, L.stream_of(out)))
+
+    if args.blocks_per_row:
+        rows = torch.arange(nb, device=dev)
+        series = {}
+        for n in (int(x) for x in args.blocks_per_row.split(",")):
+            m = torch.zeros(nb, nb, dtype=torch.bool, device=dev)
+            for j in range(n):
+                m[rows, (rows + 7 * j) % nb] = True     # the diagonal and n - 1 more columns, 7 apart
+            m = m[None].expand(H, nb, nb).contiguous()
+            series[str(n)] = round(event_time_ms(lambda: attn_only(m), 100, 2) * 1e3, 1)
+        print(json.dumps({"workload": args.workload, "attn_kernel_us_by_blocks_per_row": series}))
+        return
 
     # ---- the timed region: exactly K steps between synchronisations -------------------------
     head_mask = masks[HEADLINE_DENSITY]
