@@ -353,8 +353,15 @@ __global__ void __launch_bounds__(256) rope_k_sum_kernel(const unsigned short* _
   constexpr int LPR = D / 8;
   constexpr int ROWS = 256 / LPR;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int chunk = blockIdx.x;
-  const int bh0 = blockIdx.y * KM_GROUP;
+  // Workgroup ids are dealt round-robin to the 8 XCDs: XCD x takes the token chunks 8*i + x, and for each of
+  // them all head groups one after the other, so that a chunk of the rotary tables (twice the bytes of the
+  // K rows of one head) crosses the fabric once per launch and is served to the other head groups by that
+  // XCD's L2.
+  const int n_hg = (BH + KM_GROUP - 1) / KM_GROUP;
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const int chunk = (j / n_hg) * 8 + xcd;
+  if (chunk >= n_chunks) return;
+  const int bh0 = (j % n_hg) * KM_GROUP;
   const int col = (t % LPR) * 8;
   float s[KM_GROUP][8];
 #pragma unroll
@@ -491,7 +498,7 @@ extern "C" int paro_rope_k_mean(const void* k, int dtype, const float* cos, cons
   float* partial = (float*)workspace;
 #define PARO_KM(DTV, DV)                                                                                        \
   do {                                                                                                          \
-    hipLaunchKernelGGL((rope_k_sum_kernel<DTV, DV>), dim3(n_chunks, ceil_div(B * H, KM_GROUP)), dim3(256), 0,   \
+    hipLaunchKernelGGL((rope_k_sum_kernel<DTV, DV>), dim3(ceil_div(n_chunks, 8) * 8 * ceil_div(B * H, KM_GROUP)), dim3(256), 0, \
                        st, (const unsigned short*)k, cos, sin, partial, B * H, H, N, n_text, n_chunks,          \
                        k_stride_b, k_stride_h, k_stride_n);                                                     \
     hipLaunchKernelGGL((k_mean_finalize_kernel<DTV, DV>), dim3(B * H), dim3(1024), 0, st, (const float*)partial, \
