@@ -85,6 +85,19 @@ def event_time_ms(fn, reps, warmup):
     return e0.elapsed_time(e1) / reps
 
 
+def event_median_ms(fn, reps):
+    """Median (and minimum) over `reps` launches, each bracketed by its own pair of events."""
+    settle(fn)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in evs)
+    return ts[len(ts) // 2], ts[0]
+
+
 def mfma_ceiling(lib, L, dev):
     """Sustained rate of back-to-back MFMAs alone (no memory traffic, no VALU work), 4 waves per SIMD."""
     g = torch.Generator(device=dev).manual_seed(0)
@@ -299,6 +312,10 @@ def main():
             "pct_mfma_peak_kernel": round(100 * ex_ops / (t_kern * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 2),
             "kept_blocks": int(masks[d].sum()) * B,
         }
+        if d == HEADLINE_DENSITY:   # per-launch events (they add ~1 % between launches): median and minimum
+            med, mn = event_median_ms(lambda: attn_only(masks[d]), reps)
+            dens[str(d)]["attn_kernel_ms_median"] = round(med, 4)
+            dens[str(d)]["attn_kernel_ms_min"] = round(mn, 4)
     if not args.headline_only:
         # the same number of blocks per row as one contiguous run round the diagonal (not a benchmark
         # configuration: it shows what the mask FAMILY costs when a head's K8 + V8 exceed the L2)
