@@ -69,6 +69,9 @@ constexpr int S_MAGIC_BITS = 0x4B400000;  // float 1.5 * 2^23
 constexpr float S_MAGIC_F = 12582912.0f;
 constexpr int FP8_ONES = 0x38383838;  // four e4m3 1.0
 constexpr float FAST_EXP_SHIFT = -0.35f;  // centres the linear-mantissa error of the fast exponential
+// fast path: the real-valued byte b becomes the 16-bit field round((b + 0.5) * 256), whose HIGH byte is
+// round(b); the field is bounded by 0x7FFF, so the byte is bounded by 0x7F
+constexpr float FAST_FIELD_SCALE = 256.0f / 32767.0f;
 
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
@@ -96,15 +99,6 @@ __device__ __forceinline__ int cvt_pknorm_i16(float a, float b) {
   // (the builtin, not inline assembly: between two assembly statements the compiler assumes the worst
   // hazard and pads with s_nop)
   return __builtin_bit_cast(int, __builtin_amdgcn_cvt_pknorm_i16(a, b));
-}
-
-// field-wise maximum of three words of two non-negative 16-bit integers each: on such bit patterns
-// (small ones are half-precision denormals, 0x7C01.. are NaNs, which propagate) the packed
-// half-precision maximum orders like the integers, and a NaN still reads as "large"
-__device__ __forceinline__ int pk_max3_fields(int a, int b, int c) {
-  int r;
-  asm("v_pk_maximum3_f16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
 }
 
 __device__ __forceinline__ float partner_max(float x) {
@@ -453,9 +447,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     // scale of this block and what follows from it and from the current maximum alone
     const float c = c_cur;
     const float nmc = -S_MAGIC_F * c;
-    const float c8 = (8.0f / 32767.0f) * c;
+    const float c8 = (8.0f * FAST_FIELD_SCALE) * c;
     float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
-    float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: byte = (8*(t + 7) + shift) / 32767
+    float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: field = (8*(t + 7) + shift + 0.5) * 256 / 32767
 
     float s[2][16];
 #pragma unroll
@@ -510,7 +504,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       m_i = m_new;
       m_thr = m_new + P_HEADROOM;
       m_off = P_EXP_OFFSET - m_new;
-      m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT) * (1.0f / 32767.0f);
+      m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT + 0.5f) * FAST_FIELD_SCALE;
       bias = fmaf(-S_MAGIC_F, c, m_off);
       bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
       if constexpr (LSE) d_exact *= alpha;
@@ -529,55 +523,62 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       // Fast path: the e4m3 byte of 2^t is built directly: byte = round(8*(t + 7) + FAST_EXP_SHIFT), i.e.
       // exponent field floor(t)+7 and a mantissa that interpolates 2^frac(t) linearly between powers of
       // two (at most 6 % off, shifted to be centred).  Per word of four weights: four fmas (the affine
-      // map pre-divided by 32767, result clamped to [0,1], which sends masked and underflowing elements to
-      // 0), two v_cvt_pknorm_i16_f32 (each rounds two values to 16-bit integer fields) and one shift-or
-      // that interleaves the two pairs into bytes.  Instead of fma + v_exp_f32 + half a packed FP8
-      // conversion per weight.  Word r = word r%4 of row tile r/4.
+      // map scaled so that the byte lands in the HIGH half of a 16-bit field, result clamped to [0,1], which
+      // sends masked and underflowing elements to 0 and bounds the field by 0x7FFF, the byte by 0x7F), two
+      // v_cvt_pknorm_i16_f32 (each rounds two values to 16-bit fields) and one v_perm_b32 that gathers the
+      // four high bytes.  Instead of fma + v_exp_f32 + half a packed FP8 conversion per weight.
+      // Word r = word r%4 of row tile r/4.
       //
-      // It is optimistic about the maximum: the weights are computed with the running maximum as it
-      // is, and a packed 3-input maximum per word keeps the largest field seen.  A field above 126
-      // (the code of 448, the largest e4m3 value; fields cannot exceed 0x7FFF) means some score was more
-      // than 3.8 octaves above the running maximum: only then, and on the first block, is the block
-      // maximum searched (17 v_max3 otherwise spent on every block), the maximum refreshed and the
+      // It is optimistic about the maximum: the weights are computed with the running maximum as it is.
+      // A weight above 448, the largest e4m3 value (a score more than 3.8 octaves above the running
+      // maximum), comes out as the byte 0x7F, which is the e4m3 NaN: the row sums, taken by the matrix pipe
+      // from the same bytes BEFORE anything else uses them, turn NaN in that column, and only then is the
+      // block maximum searched (17 v_max3 otherwise spent on every block), the maximum refreshed and the
       // eight words computed again (the scores are still in `acc`: the next block's S^T is issued below).
-      auto fast_words = [&](int& ovf) {
+      // Nothing is spent on tracking in the common case, and O never sees a NaN.
+      auto fast_words = [&]() {
         float u_cur[4], u_nxt[4];
 #pragma unroll
         for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], c8, bias8);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
-          // the fmas of the next word are issued behind this word's conversions: every conversion finds
-          // its input ready, and the shift-or is not the instruction right behind the conversion it reads
-          // (a packed 16-bit result needs one wait state before a full-register read)
+          // the fmas of the next word are issued between this word's conversions: every conversion
+          // finds its input ready
           const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
-          const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
           if (rn < 8) {
             u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
             u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8, bias8);
           }
+          const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
           __builtin_amdgcn_sched_barrier(0);
-          const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
           if (rn < 8) {
             u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
             u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8, bias8);
           }
+          const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
           __builtin_amdgcn_sched_barrier(0);
-          pf[r] = (hi << 8) | lo;   // v_lshl_or_b32: the fields of hi move into the odd bytes
-          ovf = pk_max3_fields(ovf, lo, hi);
+          // bytes 1, 3 of lo (weights 0, 2) and of hi (weights 1, 3), in weight order
+          pf[r] = (int)__builtin_amdgcn_perm((unsigned)hi, (unsigned)lo, 0x07030501u);
 #pragma unroll
           for (int q = 0; q < 4; q++) u_cur[q] = u_nxt[q];
           __builtin_amdgcn_sched_barrier(0);
         }
       };
-      int ovf = 0;
-      fast_words(ovf);
-      const unsigned top = max((unsigned)ovf & 0xffffu, (unsigned)ovf >> 16);
-      if (it == 0 || __ballot(top > 126u) != 0ull) {
+      fast_words();
+      v4f d_new = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
+      // the fragment reads of the matrix phase are issued here: they cover the latency of the product above
+      __builtin_amdgcn_sched_barrier(0);
+      read_k_frags(sk1);
+      if constexpr (D == 64) read_v_frags(sv);
+      __builtin_amdgcn_sched_barrier(0);
+      // (the first block has no maximum yet; a NaN byte in column j makes every entry of column j NaN)
+      if (it == 0 || __ballot(d_new[0] != d_new[0]) != 0ull) {
         apply_refresh(block_max());
-        int ovf2 = 0;
-        fast_words(ovf2);
+        fast_words();
+        d_new = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);
       }
+      d_acc = d_new;
     } else {
       // Exact path: lazy refresh decided up front from the block maximum (P~ <= 2^(OFFSET + HEADROOM)),
       // then P~ = e4m3_rne(2^(S*c - m + OFFSET)): hardware exponential and the packed FP8 conversion
@@ -605,8 +606,10 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     //    block's P.V and row sums, which run on under that VALU phase
     // (fetching the K fragments at the head of the iteration instead, so that they arrive under the VALU
     // phase, measured 2 % slower at D = 128, 7 % with the dense mask)
-    read_k_frags(sk1);
-    if constexpr (D == 64) read_v_frags(sv);
+    if constexpr (EXACT) {   // (the fast path has issued these reads already)
+      read_k_frags(sk1);
+      if constexpr (D == 64) read_v_frags(sv);
+    }
     __builtin_amdgcn_sched_barrier(0);
     qk_mfma();
     __builtin_amdgcn_sched_barrier(0);
@@ -615,8 +618,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       read_v_frags(sv);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // (fast path: the row sums have been taken above)
 #pragma unroll
-    for (int i = 0; i < N_PV; i++) pv_one(pf, i);
+    for (int i = 0; i < (EXACT ? N_PV : DT_TILES); i++) pv_one(pf, i);
     __builtin_amdgcn_sched_barrier(0);
     if (it + 1 < cnt) dump_s(kb_1);
 
