@@ -17,8 +17,8 @@
 // chunks XOR-swizzled against bank conflicts) and V8 (already in fragment order) tiles come in by
 // LDS-DMA through a ring of three (D = 64) or two (D = 128) stages, and the loop is software-
 // pipelined: while the softmax weights of block i are computed on the VALU, the tiles of the next
-// blocks are in flight, and the MFMAs of P.V(i-1) and S^T(i+1) are issued one at a time from inside
-// the VALU stream.  One barrier per block.
+// blocks are in flight; then the MFMAs of S^T(i+1) and P.V(i) are issued back to back and run on under
+// the VALU phase of block i+1.  One barrier per block.
 //
 // Workgroups are renumbered so that each of the 8 XCDs walks a contiguous range of (batch, head,
 // q-block): the K8/V8 of the one or two heads an XCD is working on stay resident in its own L2.
@@ -332,8 +332,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   // (not in the D = 128 variants with exact exponentials, which have no 16 registers to spare)
   if constexpr (D == 64 || (!EXACT && !LSE && !DUMP)) asm volatile("" : "+v"(magic));
   v16i acc[2];
-  // the MFMAs are issued one at a time from inside the VALU stream (see step below): a wave that
-  // issues them back to back sits blocked behind the matrix pipe for their whole duration
+  // (a wave that issues MFMAs back to back sits blocked behind the matrix pipe for their whole duration;
+  // the other waves of the SIMD run their VALU phases meanwhile, see step below)
   auto qk_one = [&](int idx) {
     const int mt = idx / KS, ks = idx % KS;  // idx = mt * KS + ks, ks ascending per mt (alternating the row
                                              // tiles instead measured the same)
