@@ -335,8 +335,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   // (a wave that issues MFMAs back to back sits blocked behind the matrix pipe for their whole duration;
   // the other waves of the SIMD run their VALU phases meanwhile, see step below)
   auto qk_one = [&](int idx) {
-    const int mt = idx / KS, ks = idx % KS;  // idx = mt * KS + ks, ks ascending per mt (alternating the row
-                                             // tiles instead measured the same)
+    const int mt = idx / KS, ks = idx % KS;  // idx = mt * KS + ks
     if (ks == 0) acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[mt], qf[0], magic, 0, 0, 0);
     else acc[mt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kfrag[ks * 2 + mt], qf[ks], acc[mt], 0, 0, 0);
   };
@@ -611,11 +610,22 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       if constexpr (D == 64) read_v_frags(sv);
     }
     __builtin_amdgcn_sched_barrier(0);
-    qk_mfma();
-    __builtin_amdgcn_sched_barrier(0);
-    // (D = 128: the V fragments go into the registers the K fragments have just left)
     if constexpr (D == 128) {
-      read_v_frags(sv);
+      // the V fragments are fetched while the S^T products issue: after the two products of k-step ks the K
+      // fragments of that step are dead, and two V pieces take their place (+1-2 % against fetching all
+      // eight pieces after the last product)
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        qk_one(0 * KS + ks);
+        qk_one(1 * KS + ks);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+          vfrag[ks][mt] = *reinterpret_cast<const v4i*>(smem + sv * Lds::VTILE + vr_base + (ks * 2 + mt) * 1024);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      qk_mfma();
       __builtin_amdgcn_sched_barrier(0);
     }
     // (fast path: the row sums have been taken above)
