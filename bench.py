@@ -85,6 +85,32 @@ def event_time_ms(fn, reps, warmup):
     return e0.elapsed_time(e1) / reps
 
 
+def proxy_ceiling(lib, L, dev):
+    """The attention loop body at D = 64 as a memory-free proxy, then with its data movement added level by
+    level (paro_diag_attn_proxy): where the figure drops is what separates the kernel from the matrix pipe."""
+    g = torch.Generator(device=dev).manual_seed(0)
+    operands = torch.randint(-2 ** 31, 2 ** 31 - 1, (16384,), generator=g, device=dev, dtype=torch.int64).to(torch.int32)
+    ntiles = 278    # K8 + V8 of one CogVideoX head: 2.3 MB, stays in the L2
+    tiles = torch.randint(0, 256, (ntiles * 8192,), generator=g, device=dev, dtype=torch.int16).to(torch.uint8)
+    tiles[(tiles & 0x7F) == 0x7F] &= 0xFE     # no e4m3 NaN codes: the fp32 accumulators stay finite
+    wgs, iters = 1536, 4000     # 6 workgroups of two waves per CU = 3 waves per SIMD
+    sink = torch.empty(wgs * 128, dtype=torch.float32, device=dev)
+    ops = lib.paro_diag_attn_proxy_ops(wgs, iters)
+    names = ["0: matrix + vector instructions, operands in registers",
+             "1: + K/V fragments read from LDS every iteration (operands toggle)",
+             "2: + four LDS-DMA tile loads per wave and iteration (L2-resident, scattered order)",
+             "3: + one barrier per iteration"]
+    out = {"workgroups": wgs, "iterations": iters, "ops_per_launch": ops, "levels": {}}
+    for level, name in enumerate(names):
+        fn = lambda: L.check(lib.paro_diag_attn_proxy(level, L.ptr(operands), L.ptr(tiles), L.ptr(sink), wgs, iters,
+                                                      ntiles, L.stream_of(sink)))
+        t = event_time_ms(fn, 10, 2)
+        out["levels"][name] = {"ms": round(t, 4), "ns_per_wave_iteration_per_simd": round(t * 1e6 / iters / 3, 1),
+                               "counted_tops": round(ops / (t * 1e-3) / 1e12, 1),
+                               "pct_of_nominal_peak": round(100 * ops / (t * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 1)}
+    return out
+
+
 def event_median_ms(fn, reps):
     """Median (and minimum) over `reps` launches, each bracketed by its own pair of events."""
     settle(fn)
@@ -201,6 +227,9 @@ def main():
                     help="only time back-to-back MFMAs (int8 and fp8, random and zero operands): what the matrix pipe "
                          "sustains on this box, the ceiling of any kernel built on it.  Prints its own JSON line.")
     ap.add_argument("--exact-exp", action="store_true", help="attention kernel with exact exponentials (flag PARO_ATTN_EXACT_EXP)")
+    ap.add_argument("--proxy-ceiling", action="store_true",
+                    help="measurement aid: instead of the benchmark, time a proxy of the attention loop body (D = 64) "
+                         "without memory traffic, then with LDS fragment reads, tile DMA and the barrier added in turn")
     ap.add_argument("--blocks-per-row", default=None, metavar="LIST",
                     help="measurement aid: instead of the benchmark, time the attention kernel with masks that keep "
                          "exactly n blocks in every row, for every n of the comma-separated list (0,1,2,4,...): what a "
@@ -227,6 +256,9 @@ def main():
     lib = L.load()
     if args.mfma_ceiling:
         print(json.dumps(mfma_ceiling(lib, L, dev)))
+        return
+    if args.proxy_ceiling:
+        print(json.dumps(proxy_ceiling(lib, L, dev)))
         return
     wl = synth.WORKLOADS[args.workload]
     global HEADLINE_DENSITY, DENSITIES

@@ -320,6 +320,17 @@ int paro_mask_unpack(const uint8_t* bits, uint8_t* mask, int64_t n, void* stream
 int64_t paro_diag_mfma_loop_ops(int kind, int workgroups, int iters);
 int paro_diag_mfma_loop(int kind, const void* operands, float* sink, int workgroups, int iters, void* stream);
 
+/* Measurement aid, no counterpart in the reference: a proxy of the attention loop body at D = 64 (the same
+ * matrix and vector instructions per wave and iteration, workgroups of two waves) at four levels: 0 operands in
+ * registers, 1 + K/V fragments read from LDS every iteration, 2 + the four LDS-DMA tile loads per wave and
+ * iteration, 3 + one barrier per iteration.  operands: 16384 int32 of device memory (random bytes); tiles:
+ * ntiles * 8192 bytes (random e4m3 bytes other than the NaN codes), ntiles <= 65535; sink: workgroups * 128 floats.
+ * paro_diag_attn_proxy_ops() = operations one launch is credited with, counted as the attention kernel counts
+ * a block.  Used by bench.py --proxy-ceiling. */
+int64_t paro_diag_attn_proxy_ops(int workgroups, int iters);
+int paro_diag_attn_proxy(int level, const void* operands, const void* tiles, float* sink, int workgroups, int iters,
+                         int ntiles, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

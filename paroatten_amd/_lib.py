@@ -71,6 +71,8 @@ SIGNATURES = {
                                        _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
     "paro_diag_mfma_loop_ops": (c_int64, [_I, _I, _I]),
     "paro_diag_mfma_loop": (c_int, [_P, _P, _P, _I, _I, _P]),
+    "paro_diag_attn_proxy_ops": (c_int64, [_I, _I]),
+    "paro_diag_attn_proxy": (c_int, [_I, _P, _P, _P, _I, _I, _I, _P]),
     "paro_sub_mean": (c_int, [_P, _I, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
 }
 

@@ -569,7 +569,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       // the fragment reads of the matrix phase are issued here: they cover the latency of the product above
       __builtin_amdgcn_sched_barrier(0);
       read_k_frags(sk1);
+#ifndef V_AFTER_QK
       if constexpr (D == 64) read_v_frags(sv);
+#endif
       __builtin_amdgcn_sched_barrier(0);
       // (the first block has no maximum yet; a NaN byte in column j makes every entry of column j NaN)
       if (it == 0 || __ballot(d_new[0] != d_new[0]) != 0ull) {
@@ -607,7 +609,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     // phase, measured 2 % slower at D = 128, 7 % with the dense mask)
     if constexpr (EXACT) {   // (the fast path has issued these reads already)
       read_k_frags(sk1);
+#ifndef V_AFTER_QK
       if constexpr (D == 64) read_v_frags(sv);
+#endif
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (D == 128) {
@@ -627,6 +631,10 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     } else {
       qk_mfma();
       __builtin_amdgcn_sched_barrier(0);
+#ifdef V_AFTER_QK
+      read_v_frags(sv);
+      __builtin_amdgcn_sched_barrier(0);
+#endif
     }
     // (fast path: the row sums have been taken above)
 #pragma unroll
