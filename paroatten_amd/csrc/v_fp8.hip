@@ -55,7 +55,9 @@ __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __re
       v4i raw[VS_BATCH];
 #pragma unroll
       for (int u = 0; u < VS_BATCH; u++)
-        raw[u] = *reinterpret_cast<const v4i*>(vb + (int64_t)(tok0 + r + u * ROWS) * vs_n);
+        // (non-temporal: measured 3-5 us faster per launch of the entry point and of the per-layer sequence
+        // than ordinary loads, although the packing pass reads the same tensor right afterwards)
+        raw[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(vb + (int64_t)(tok0 + r + u * ROWS) * vs_n));
 #pragma unroll
       for (int u = 0; u < VS_BATCH; u++) take(raw[u]);
     }
