@@ -573,8 +573,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       if constexpr (D == 64) read_v_frags(sv);
 #endif
       __builtin_amdgcn_sched_barrier(0);
-      // (the first block has no maximum yet; a NaN byte in column j makes every entry of column j NaN)
-      if (it == 0 || __ballot(d_new[0] != d_new[0]) != 0ull) {
+      // (the first block has no maximum yet.  Lane j < 16 holds the sums of q-rows j and j + 16 in d_new[0]
+      // and d_new[1]; a NaN byte of either row makes its own sum NaN whatever the hardware makes of 0 x NaN)
+      if (it == 0 || __ballot(__builtin_isunordered(d_new[0], d_new[1])) != 0ull) {
         apply_refresh(block_max());
         fast_words();
         d_new = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pf, d_acc, 0, 0, 0, 0, 0, 0);

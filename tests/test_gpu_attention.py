@@ -216,8 +216,8 @@ def _ramp_case(B, H, N, D, dtype, seed, pattern):
                                                     ("spike", False, 0.5), ("spike", True, 1.0)])
 def test_fast_path_maximum_recovery(dev, D, pattern, causal, density):
     """The default (fast) softmax path computes a block's weights against the running maximum as it is
-    and only afterwards notices, from the largest 16-bit field it built, that a score was more than the
-    FP8 headroom above it; it then refreshes the maximum and recomputes the block.  Here that happens in
+    and only afterwards notices, from a NaN in the row sums of the bytes it built, that a score was more
+    than the FP8 headroom above it; it then refreshes the maximum and recomputes the block.  Here that happens in
     block after block (every row, dense, sparse and causal masks): the output must be finite and match
     both the oracle and the exact-exponential path."""
     import paroatten_amd as P
@@ -256,6 +256,46 @@ def test_fast_path_maximum_recovery(dev, D, pattern, causal, density):
     close(o_fast, o_ref)
     close(o_exact, o_ref)
     close(o_fast, o_exact)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("row", [3, 20, 37, 59])
+def test_fast_path_overflow_of_a_single_row(dev, D, row):
+    """One q-row of one q-block alone meets a key far above its running maximum, late in its row: the row sits
+    in the lower or upper half of either wave's 32 rows (the row sums of rows j and j + 16 share a lane of the
+    row-sum product, and the overflow test has to see each of them).  Every other row must be untouched by
+    the refresh that this row forces on its wave (same result as the exact path to the usual tolerance)."""
+    import paroatten_amd as P
+    B, H, N = 1, 1, 640
+    nb = N // 64
+    q, k, v = synth.make_qkv(B, H, N, D, torch.float16, seed=row, k_bias_std=0.0)
+    g = torch.Generator().manual_seed(1000 + row)
+    w = torch.randn(D, generator=g)
+    w = w / w.norm()
+    qf, kf = q.float() * 0.3, k.float() * 0.3
+    qrow, key = 64 * 3 + row, 64 * 8 + 11            # q-block 3, key block 8 of 10
+    sm = D ** -0.5
+    qf[0, 0, qrow] = 4.0 * w
+    kf[0, 0, key] = (14.0 / (4.0 * sm)) * w            # 14 nats = 20 octaves above the rest, for this row only
+    q, k = qf.to(torch.float16), kf.to(torch.float16)
+    mask = torch.ones(H, nb, nb, dtype=torch.bool)
+    q8, qs, k8, ks = O.per_warp_int8(q, k, BLKQ=64, WARPQ=32, BLKK=64)
+    o_ref, _ = O.sparse_attention(q8, k8, v, qs, ks, mask[None], sm, out_dtype=torch.float32)
+    a_ref, _ = O.sparse_attention(q8, k8, v.abs(), qs, ks, mask[None], sm, out_dtype=torch.float32)
+    kw = dict(smooth_k=False)
+    o_fast = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), **kw).cpu()
+    o_exact = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), exact_exp=True, **kw).cpu()
+    assert torch.isfinite(o_fast.float()).all()
+    for got in (o_fast, o_exact):
+        e = (got.float() - o_ref).abs()
+        assert bool((e <= ATOL + 0.125 * a_ref).all()), float((e - 0.125 * a_ref).max())
+        assert cosine(got, o_ref) >= COS
+    # the row itself is dominated by the one key: its output is that key's V row to FP8 accuracy
+    dom = o_fast[0, 0, qrow].float()
+    assert cosine(dom, v[0, 0, key].float()) >= 0.995
+    # and the other rows of its q-block agree with the exact path like any other row
+    others = [r for r in range(64 * 3, 64 * 4) if r != qrow]
+    assert cosine(o_fast[0, 0, others], o_exact[0, 0, others]) >= COS
 
 
 @pytest.mark.parametrize("D,H,N", [(128, 8, 16384), (64, 16, 12352)])
