@@ -85,29 +85,75 @@ def event_time_ms(fn, reps, warmup):
     return e0.elapsed_time(e1) / reps
 
 
-def proxy_ceiling(lib, L, dev):
+def load_diag():
+    """libparoatten_diag.so (include/paroatten_diag.h): the measurement aids, outside the product library."""
+    import ctypes
+    from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "paroatten_amd", "lib", "libparoatten_diag.so")
+    if not os.path.exists(path):
+        raise SystemExit(f"{path} is not built: run `python paroatten_amd/build.py`")
+    d = ctypes.CDLL(path)
+    P, I = c_void_p, c_int
+    for name, res, args in (("paro_diag_last_error", c_char_p, []),
+                            ("paro_diag_mfma_loop_ops", c_int64, [I, I, I]),
+                            ("paro_diag_mfma_loop", I, [I, P, P, I, I, P]),
+                            ("paro_diag_attn_proxy_ops", c_int64, [I, I]),
+                            ("paro_diag_attn_proxy", I, [I, P, P, P, I, I, I, P]),
+                            ("paro_diag_attn_proxy_w64_ops", c_int64, [I, I]),
+                            ("paro_diag_attn_proxy_w64", I, [I, P, P, P, P, I, I, I, P])):
+        fn = getattr(d, name)
+        fn.restype, fn.argtypes = res, args
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(d.paro_diag_last_error().decode())
+    d.ok = ok
+    return d
+
+
+def proxy_ceiling(diag, L, dev):
     """The attention loop body at D = 64 as a memory-free proxy, then with its data movement added level by
-    level (paro_diag_attn_proxy): where the figure drops is what separates the kernel from the matrix pipe."""
+    level: first as the two-waves-per-q-block kernel arranges it (paro_diag_attn_proxy), then as the
+    one-wave-per-q-block kernel does (paro_diag_attn_proxy_w64).  Where the figure drops is what separates a
+    kernel from the matrix pipe; the second set also reads the shader clock inside the kernel."""
     g = torch.Generator(device=dev).manual_seed(0)
     operands = torch.randint(-2 ** 31, 2 ** 31 - 1, (16384,), generator=g, device=dev, dtype=torch.int64).to(torch.int32)
     ntiles = 278    # K8 + V8 of one CogVideoX head: 2.3 MB, stays in the L2
     tiles = torch.randint(0, 256, (ntiles * 8192,), generator=g, device=dev, dtype=torch.int16).to(torch.uint8)
     tiles[(tiles & 0x7F) == 0x7F] &= 0xFE     # no e4m3 NaN codes: the fp32 accumulators stay finite
     wgs, iters = 1536, 4000     # 6 workgroups of two waves per CU = 3 waves per SIMD
-    sink = torch.empty(wgs * 128, dtype=torch.float32, device=dev)
-    ops = lib.paro_diag_attn_proxy_ops(wgs, iters)
+    sink = torch.empty(2048 * 128, dtype=torch.float32, device=dev)
+    ops = diag.paro_diag_attn_proxy_ops(wgs, iters)
     names = ["0: matrix + vector instructions, operands in registers",
              "1: + K/V fragments read from LDS every iteration (operands toggle)",
              "2: + four LDS-DMA tile loads per wave and iteration (L2-resident, scattered order)",
              "3: + one barrier per iteration"]
-    out = {"workgroups": wgs, "iterations": iters, "ops_per_launch": ops, "levels": {}}
+    out = {"workgroups": wgs, "iterations": iters, "ops_per_launch": ops, "levels": {}, "one_wave_per_q_block": {}}
     for level, name in enumerate(names):
-        fn = lambda: L.check(lib.paro_diag_attn_proxy(level, L.ptr(operands), L.ptr(tiles), L.ptr(sink), wgs, iters,
-                                                      ntiles, L.stream_of(sink)))
+        fn = lambda: diag.ok(diag.paro_diag_attn_proxy(level, L.ptr(operands), L.ptr(tiles), L.ptr(sink), wgs, iters,
+                                                       ntiles, L.stream_of(sink)))
         t = event_time_ms(fn, 10, 2)
         out["levels"][name] = {"ms": round(t, 4), "ns_per_wave_iteration_per_simd": round(t * 1e6 / iters / 3, 1),
                                "counted_tops": round(ops / (t * 1e-3) / 1e12, 1),
                                "pct_of_nominal_peak": round(100 * ops / (t * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 1)}
+    # one wave = 64 q-rows: 2048 one-wave workgroups = 2 waves per SIMD, 2000 iterations of both halves
+    wgs2, iters2 = 2048, 2000
+    ops2 = diag.paro_diag_attn_proxy_w64_ops(wgs2, iters2)
+    clk = torch.zeros(2, dtype=torch.int64, device=dev)
+    names2 = ["0: operands in registers", "1: + 8 fragment reads per block (each feeds two products)",
+              "2: + 8 LDS-DMA tile loads per block instead (no reads)", "3: + reads and tile loads",
+              "4: as 3, V straight from memory into registers (no LDS round trip for V)"]
+    for variant, name in enumerate(names2):
+        fn = lambda: diag.ok(diag.paro_diag_attn_proxy_w64(variant, L.ptr(operands), L.ptr(tiles), L.ptr(sink), L.ptr(clk),
+                                                           wgs2, iters2, ntiles, L.stream_of(sink)))
+        t = event_time_ms(fn, 10, 2)
+        cyc, ticks = (int(x) for x in clk.tolist())
+        ghz = cyc / (ticks * 10.0) if ticks else 0.0
+        ns = t * 1e6 / iters2 / 2 / 2     # per 32-row half-block and SIMD (two waves per SIMD, two halves per iteration)
+        out["one_wave_per_q_block"][name] = {
+            "ms": round(t, 4), "ns_per_32_row_block_per_simd": round(ns, 1), "shader_clock_ghz": round(ghz, 3),
+            "cycles_per_32_row_block_per_simd": round(ns * ghz, 1),
+            "pct_of_nominal_peak": round(100 * ops2 / (t * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 1)}
     return out
 
 
@@ -124,7 +170,7 @@ def event_median_ms(fn, reps):
     return ts[len(ts) // 2], ts[0]
 
 
-def mfma_ceiling(lib, L, dev):
+def mfma_ceiling(diag, L, dev):
     """Sustained rate of back-to-back MFMAs alone (no memory traffic, no VALU work), 4 waves per SIMD."""
     g = torch.Generator(device=dev).manual_seed(0)
     rnd = torch.randint(-2 ** 31, 2 ** 31 - 1, (64 * 16,), generator=g, device=dev, dtype=torch.int64).to(torch.int32)
@@ -137,9 +183,9 @@ def mfma_ceiling(lib, L, dev):
     out = {"metric": "sustained MFMA rate, back-to-back instructions only", "unit": "TOP/s",
            "peak_nominal": PEAK_MFMA_TOPS, "workgroups": wgs, "iters": iters}
     for kind, kname in ((0, "int8_32x32x32"), (1, "fp8_32x32x64")):
-        ops = lib.paro_diag_mfma_loop_ops(kind, wgs, iters)
+        ops = diag.paro_diag_mfma_loop_ops(kind, wgs, iters)
         for oname, buf in (("random", rnd), ("zero", zero)):
-            fn = lambda: L.check(lib.paro_diag_mfma_loop(kind, L.ptr(buf), L.ptr(sink), wgs, iters, L.stream_of(sink)))
+            fn = lambda: diag.ok(diag.paro_diag_mfma_loop(kind, L.ptr(buf), L.ptr(sink), wgs, iters, L.stream_of(sink)))
             t = event_time_ms(fn, 10, 2)
             out[f"{kname}_{oname}"] = {"ms": round(t, 3), "tops": round(ops / (t * 1e-3) / 1e12, 1),
                                        "frac_nominal": round(ops / (t * 1e-3) / 1e12 / PEAK_MFMA_TOPS, 3)}
@@ -227,6 +273,9 @@ def main():
                     help="only time back-to-back MFMAs (int8 and fp8, random and zero operands): what the matrix pipe "
                          "sustains on this box, the ceiling of any kernel built on it.  Prints its own JSON line.")
     ap.add_argument("--exact-exp", action="store_true", help="attention kernel with exact exponentials (flag PARO_ATTN_EXACT_EXP)")
+    ap.add_argument("--two-waves", action="store_true",
+                    help="attention kernel with two waves per q-block (flag PARO_ATTN_TWO_WAVES) also at head size 64, "
+                         "where the default is the one-wave-per-q-block kernel")
     ap.add_argument("--proxy-ceiling", action="store_true",
                     help="measurement aid: instead of the benchmark, time a proxy of the attention loop body (D = 64) "
                          "without memory traffic, then with LDS fragment reads, tile DMA and the barrier added in turn")
@@ -255,10 +304,10 @@ def main():
     torch.cuda.set_device(dev)
     lib = L.load()
     if args.mfma_ceiling:
-        print(json.dumps(mfma_ceiling(lib, L, dev)))
+        print(json.dumps(mfma_ceiling(load_diag(), L, dev)))
         return
     if args.proxy_ceiling:
-        print(json.dumps(proxy_ceiling(lib, L, dev)))
+        print(json.dumps(proxy_ceiling(load_diag(), L, dev)))
         return
     wl = synth.WORKLOADS[args.workload]
     global HEADLINE_DENSITY, DENSITIES
@@ -292,7 +341,7 @@ def main():
         aq8, ak8, av8 = torch.zeros_like(q8), torch.zeros_like(k8), torch.zeros_like(v8)
     else:
         aq8, ak8, av8 = q8, k8, v8
-    attn_flags = L.PARO_ATTN_EXACT_EXP if args.exact_exp else 0
+    attn_flags = (L.PARO_ATTN_EXACT_EXP if args.exact_exp else 0) | (L.PARO_ATTN_TWO_WAVES if args.two_waves else 0)
 
     def attn_only(mask):  # the attention kernel alone (for the roofline)
         L.check(lib.paro_attn_sparse_fwd(

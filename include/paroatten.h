@@ -47,6 +47,9 @@ extern "C" {
                                  PARO_ATTN_PACING=0/1 overrides that default).  Scattered masks on long sequences gain
                                  (Wan 720p, uniformly random blocks: 26 -> 35 % of the MFMA peak, 3.3x fewer L2 fills);
                                  masks made of one contiguous run per row lose a few per cent. */
+#define PARO_ATTN_TWO_WAVES 8 /* kernel form, results are bit-identical either way: two waves per 64-row q-block
+                                 (32 q-rows each) also where the library would pick the one-wave-per-q-block
+                                 kernel (head size 64, no lse, plain launch), which is the faster of the two there */
 
 /* Version of this ABI (bumped when a signature changes). */
 int paro_abi_version(void);
@@ -308,28 +311,6 @@ int paro_channel_quant_fp8(const void* in, int dtype, uint8_t* out, float* mean,
 int64_t paro_mask_bits_bytes(int64_t n);
 int paro_mask_pack(const uint8_t* mask, uint8_t* bits, int64_t n, void* stream);
 int paro_mask_unpack(const uint8_t* bits, uint8_t* mask, int64_t n, void* stream);
-
-/* ---------------------------------------------------------------------------------------------
- * Measurement aid (no counterpart in the reference): `workgroups` workgroups of four waves each issue
- * `iters` x 4 back-to-back MFMAs of the kind the attention kernel uses (kind 0: v_mfma_i32_32x32x32_i8,
- * kind 1: v_mfma_f32_32x32x64_f8f6f4 on e4m3 operands) with nothing else in the loop.  operands: 4 KiB of
- * device memory (64 lanes x 16 words) that every wave takes its A / B registers from (random bytes or
- * zeros); sink: one float per wave (workgroups * 4).  paro_diag_mfma_loop_ops() = operations one launch
- * executes.  Timed by the caller, it gives what the matrix pipe sustains on the GPU at hand.
- * ------------------------------------------------------------------------------------------- */
-int64_t paro_diag_mfma_loop_ops(int kind, int workgroups, int iters);
-int paro_diag_mfma_loop(int kind, const void* operands, float* sink, int workgroups, int iters, void* stream);
-
-/* Measurement aid, no counterpart in the reference: a proxy of the attention loop body at D = 64 (the same
- * matrix and vector instructions per wave and iteration, workgroups of two waves) at four levels: 0 operands in
- * registers, 1 + K/V fragments read from LDS every iteration, 2 + the four LDS-DMA tile loads per wave and
- * iteration, 3 + one barrier per iteration.  operands: 16384 int32 of device memory (random bytes); tiles:
- * ntiles * 8192 bytes (random e4m3 bytes other than the NaN codes), ntiles <= 65535; sink: workgroups * 128 floats.
- * paro_diag_attn_proxy_ops() = operations one launch is credited with, counted as the attention kernel counts
- * a block.  Used by bench.py --proxy-ceiling. */
-int64_t paro_diag_attn_proxy_ops(int workgroups, int iters);
-int paro_diag_attn_proxy(int level, const void* operands, const void* tiles, float* sink, int workgroups, int iters,
-                         int ntiles, void* stream);
 
 #ifdef __cplusplus
 }

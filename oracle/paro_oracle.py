@@ -18,9 +18,11 @@ Pinning status
   permute maps / permute_qk / permute_attn_out: pinned (torch.permute library routine, the
         reference's literal tables, inverse∘forward = id)
   rope_wan                                    : pinned (complex rotation, norm, composition)
-  rope_cog (cos/sin table convention of diffusers' get_3d_rotary_pos_embed) : the rotation
-        itself is pinned; the TABLE CONSTRUCTION is "parity unpinned" (third-party diffusers,
-        no version pinned by the reference, not importable here)
+  rope_cog (cos/sin table convention of diffusers' get_3d_rotary_pos_embed) : pinned (the
+        rotation by complex multiplication and norm preservation; the table by closed forms
+        evaluated in Python floats: 16/24/24 channel groups that each depend on one grid axis,
+        angle = pos * theta^(-2i/dim_group) on both channels of pair i, and an independent
+        second construction in paroatten_amd/rope.py compared bit for bit)
   per_channel_fp8                             : pinned against torch.float8_e4m3fn casting
   transpose_pad_permute                       : pinned (torch.transpose + pad library routines; the
         within-16 order is stated twice by the reference, as a formula in the kernel and as a
@@ -307,9 +309,10 @@ def rope_table_wan(head_dim: int, grid: Sequence[int], theta: float = 10000.0) -
 def rope_table_cog(head_dim: int, grid: Sequence[int], theta: float = 10000.0):
     """CogVideoX 3-D table in the documented diffusers convention: channels split
     t/h/w = D/4, 3D/8, 3D/8, every frequency repeated twice (repeat_interleave 2), cos/sin
-    fp32 [F*H*W, D].  PARITY UNPINNED: third-party table construction (diffusers'
-    get_3d_rotary_pos_embed, no version pinned, not importable here); the reference only
-    consumes the finished (cos, sin) pair (cogvideox.py:167-172)."""
+    fp32 [F*H*W, D].  The reference only consumes the finished (cos, sin) pair
+    (cogvideox.py:167-172); the convention (third-party diffusers get_3d_rotary_pos_embed, no
+    version pinned by the reference, not importable here) is pinned by closed forms in
+    tests/test_oracle_permute_rope.py (test_rope_cog_table_closed_form)."""
     F, Hh, W = grid
     dt, dh, dw = head_dim // 4, head_dim // 8 * 3, head_dim // 8 * 3
     af = rope_1d_freqs(dt, F, theta).repeat_interleave(2, dim=1)

@@ -22,6 +22,7 @@ PARO_ERR_HIP = -4
 PARO_ATTN_EXACT_EXP = 1
 PARO_ATTN_PACED = 2
 PARO_ATTN_UNPACED = 4
+PARO_ATTN_TWO_WAVES = 8
 
 DTYPE_CODE = {torch.float16: 0, torch.bfloat16: 1}
 
@@ -69,10 +70,6 @@ SIGNATURES = {
     "paro_transpose_pad_permute": (c_int, [_P, _P, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
     "paro_channel_quant_fp8": (c_int, [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F,
                                        _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
-    "paro_diag_mfma_loop_ops": (c_int64, [_I, _I, _I]),
-    "paro_diag_mfma_loop": (c_int, [_P, _P, _P, _I, _I, _P]),
-    "paro_diag_attn_proxy_ops": (c_int64, [_I, _I]),
-    "paro_diag_attn_proxy": (c_int, [_I, _P, _P, _P, _I, _I, _I, _P]),
     "paro_sub_mean": (c_int, [_P, _I, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _P]),
 }
 

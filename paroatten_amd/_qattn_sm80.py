@@ -31,12 +31,14 @@ def _chk(cond, msg):
         raise RuntimeError(msg)
 
 
-def _flags(exact_exp, pacing):
-    """pacing: None (the library chooses), True (PARO_ATTN_PACED) or False (PARO_ATTN_UNPACED): the launch
-    form only, results are bit-identical."""
+def _flags(exact_exp, pacing, two_waves=False):
+    """pacing: None (the library chooses), True (PARO_ATTN_PACED) or False (PARO_ATTN_UNPACED); two_waves:
+    PARO_ATTN_TWO_WAVES.  Launch and kernel form only: results are bit-identical."""
     f = _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0
     if pacing is not None:
         f |= _lib.PARO_ATTN_PACED if pacing else _lib.PARO_ATTN_UNPACED
+    if two_waves:
+        f |= _lib.PARO_ATTN_TWO_WAVES
     return f
 
 
@@ -46,7 +48,7 @@ def workspace_bytes(B, Hkv, Nk, D):
 
 def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_scale, tensor_layout, is_causal,
                                   qk_quant_gran, sm_scale, return_lse, sparse, *, smooth_v=True, exact_exp=False,
-                                  workspace=None, pacing=None):
+                                  workspace=None, pacing=None, two_waves=False):
     for t, n in ((query, "query"), (key, "key"), (value, "value"), (output, "output"),
                  (query_scale, "query_scale"), (key_scale, "key_scale")):
         _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
@@ -127,12 +129,13 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
         value.stride(0), value.stride(sh), value.stride(sn),
         output.stride(0), output.stride(sh), output.stride(sn),
         tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0,
-        _flags(exact_exp, pacing), stream_of(query))
+        _flags(exact_exp, pacing, two_waves), stream_of(query))
     return lse
 
 
 def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_scale, sm_scale, sparse,
-                          is_causal=0, return_lse=0, exact_exp=False, unpermute=None, pacing=None):
+                          is_causal=0, return_lse=0, exact_exp=False, unpermute=None, pacing=None,
+                          two_waves=False):
     """The attention kernel alone, on operands that are already in its formats (HND, contiguous):
     q8/k8 int8 [B,H,N,D] / [B,Hkv,Nk,D], v8 = FP8 tiles from paro_v_fp8_pack or the fused
     preparation, v_scale / v_mean f32 [B,Hkv,D] (v_mean None: V was not mean-smoothed).  No
@@ -165,7 +168,7 @@ def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_
         _chk(tuple(sparse.shape) == (H, nbq, nbk), f"Tensor sparse must have shape ([{B},] {H}, {nbq}, {nbk})")
         sparse_bs = 0
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q8.device) if return_lse else torch.empty(0)
-    flags = _flags(exact_exp, pacing)
+    flags = _flags(exact_exp, pacing, two_waves)
     strides = (q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
                output.stride(0), output.stride(1), output.stride(2))
     if unpermute is None:

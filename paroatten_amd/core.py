@@ -33,7 +33,7 @@ def paroattn(q, k, v, tensor_layout: str = "HND", is_causal: bool = False, sm_sc
 def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", is_causal: bool = False,
                                   qk_quant_gran: str = "per_warp", sm_scale: Optional[float] = None,
                                   return_lse: bool = False, smooth_k: bool = False, smooth_v: bool = True,
-                                  exact_exp: bool = False, **kwargs: Any):
+                                  exact_exp: bool = False, two_waves: bool = False, **kwargs: Any):
     """INT8 Q.K^T, FP8 P.V block-sparse attention.
 
     q [B,Hq,Nq,D] / k, v [B,Hkv,Nk,D] ("HND") or [B,N,H,D] ("NHD"), float16 or bfloat16, same
@@ -42,7 +42,8 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
     Returns o (q's dtype and shape) or (o, lse) with lse the natural-log sum-exp per row.
     smooth_k subtracts the per-(batch,head) token mean of K before quantisation (softmax is
     invariant to it); smooth_v does the same for V inside the FP8 conversion and adds the mean back;
-    exact_exp trades speed for fp32-evaluated softmax exponentials (see _qattn_sm80).
+    exact_exp trades speed for fp32-evaluated softmax exponentials (see _qattn_sm80); two_waves picks the
+    two-waves-per-q-block kernel where the library would take the one-wave one (bit-identical results).
     """
     dtype = q.dtype
     assert q.is_cuda, "Input tensors must be on cuda."
@@ -81,7 +82,8 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
         o = torch.empty(q.size(), dtype=dtype, device=q.device)
         lse = qattn.qk_int8_sv_f16_accum_f16_attn(q_int8, k_int8, v, o, q_scale, k_scale, layout_flag,
                                                   1 if is_causal else 0, 2, sm_scale, 1 if return_lse else 0,
-                                                  sparse, smooth_v=smooth_v, exact_exp=exact_exp)
+                                                  sparse, smooth_v=smooth_v, exact_exp=exact_exp,
+                                                  two_waves=two_waves)
         o = o[..., :head_dim_og]
         if return_lse:
             return o, lse / 1.44269504

@@ -27,91 +27,11 @@
 // (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:44-726) as instantiated by its host (:1022-1048):
 // scale indexing :100-133, mask indexing :222/:268, out-of-range columns attn_utils.cuh:355-381,
 // softmax recurrence attn_utils.cuh:383-488, normalisation :786-840, lse = log2(d) + m (:711-723).
-#include "paro_device.hpp"
+#include "attn_common.hpp"
 #include <mutex>
 #include <stdlib.h>
-#include <type_traits>
 
 namespace paro {
-
-struct AttnParams {
-  const int8_t* q8;
-  const int8_t* k8;
-  const uint8_t* v8;
-  const float* q_scale;
-  const float* k_scale;
-  const float* v_scale;
-  const float* v_mean;
-  const uint8_t* sparse;
-  void* out;
-  float* lse;
-  int32_t* s_dump;
-  int64_t sparse_bs;
-  int64_t qs_b, qs_h, qs_n;
-  int64_t ks_b, ks_h, ks_n;
-  int64_t os_b, os_h, os_n;
-  int B, H, Hkv, Nq, Nk, nbq, nbk;
-  int total;  // B*H*nbq workgroups that have work
-  float sm_scale_log2e;
-  // optional inverse permutation on the way out: q-row r of head h is stored at token
-  // n_text + unpermute(r - n_text, orders[h]) (rows below n_text stay); orders == nullptr: row r
-  const int* orders;
-  int n_text, F, Hh, W;
-  int pacing;  // +1: paced launch asked for, -1: plain launch asked for, 0: the library chooses
-};
-
-// P~ = 2^(S*c - m + P_EXP_OFFSET).  m is the running row maximum, refreshed lazily: only when a
-// block's maximum exceeds it by more than P_HEADROOM are m, O and the row sums rescaled, so that
-// P~ <= 2^(P_EXP_OFFSET + P_HEADROOM) = 2^8.75 < 448, the largest e4m3 value.
-constexpr float P_EXP_OFFSET = 5.0f;
-constexpr float P_HEADROOM = 3.75f;
-constexpr int S_MAGIC_BITS = 0x4B400000;  // float 1.5 * 2^23
-constexpr float S_MAGIC_F = 12582912.0f;
-constexpr int FP8_ONES = 0x38383838;  // four e4m3 1.0
-constexpr float FAST_EXP_SHIFT = -0.35f;  // centres the linear-mantissa error of the fast exponential
-// fast path: the real-valued byte b becomes the 16-bit field round((b + 0.5) * 256), whose HIGH byte is
-// round(b); the field is bounded by 0x7FFF, so the byte is bounded by 0x7F
-constexpr float FAST_FIELD_SCALE = 256.0f / 32767.0f;
-
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-
-// two floats -> two e4m3 bytes in the low (HI = false) or high half of a word; the other half of the
-// destination is left as it is, so a full word takes one call of each kind
-template <bool HI>
-__device__ __forceinline__ void cvt_pk_fp8(int& w, float a, float b) {
-  if constexpr (HI) asm("v_cvt_pk_fp8_f32 %0, %1, %2 op_sel:[0,0,1]" : "+v"(w) : "v"(a), "v"(b));
-  else asm("v_cvt_pk_fp8_f32 %0, %1, %2" : "=v"(w) : "v"(a), "v"(b));  // upper half: don't care, overwritten next
-}
-
-// a*b + c clamped to [0,1] (the clamp is an output modifier: no extra instruction)
-__device__ __forceinline__ float fma_clamp01(float a, float b, float c) {
-  float r;
-  asm("v_fma_f32 %0, %1, %2, %3 clamp" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
-}
-
-// two floats in [0,1] -> round(x * 32767) as two 16-bit fields (never negative, at most 0x7FFF)
-__device__ __forceinline__ int cvt_pknorm_i16(float a, float b) {
-  // (the builtin, not inline assembly: between two assembly statements the compiler assumes the worst
-  // hazard and pads with s_nop)
-  return __builtin_bit_cast(int, __builtin_amdgcn_cvt_pknorm_i16(a, b));
-}
-
-__device__ __forceinline__ float partner_max(float x) {
-  // max of own value and that of lane ^ 32: v_permlane32_swap exchanges the upper half of its
-  // first operand with the lower half of its second
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return max3(__uint_as_float(r[0]), __uint_as_float(r[1]), __uint_as_float(r[1]));
-}
-
-__device__ __forceinline__ v4i buffer_load16(__amdgpu_buffer_rsrc_t rsrc, int voffset, int soffset) {
-  // out-of-range bytes read as 0 (raw buffer, bounds-checked by the hardware)
-  return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voffset, soffset, 0));
-}
 
 template <int D> struct AttnLds {
   // LDS ring stages per operand.  D = 64: three, tiles are requested two iterations ahead.  D = 128:
@@ -134,17 +54,6 @@ template <int D> struct AttnLds {
     else return (row ^ (row >> 3)) & 7;
   }
 };
-
-// LDS-DMA: 16 bytes per lane from a buffer straight into LDS at lds_base + lane*16; no registers, no
-// ds_write; completion is counted by vmcnt
-// IMM (a compile-time constant below 4096) is added to BOTH the memory offset and the LDS address: the
-// pieces of one tile share one LDS base register (M0) and differ in IMM only
-template <int IMM>
-__device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_base, int voffset,
-                                                  int soffset) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_base, 16, voffset,
-                                           soffset, IMM, 0);
-}
 
 // Waves per SIMD the register budget is set for: the D = 64 production variants fit 168 registers.
 #define PARO_ATTN_WAVES_PER_SIMD ((D == 64 && !CAUSAL && !DUMP && !LSE) ? 3 : 2)
@@ -574,9 +483,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       // the fragment reads of the matrix phase are issued here: they cover the latency of the product above
       __builtin_amdgcn_sched_barrier(0);
       read_k_frags(sk1);
-#ifndef V_AFTER_QK
       if constexpr (D == 64) read_v_frags(sv);
-#endif
       __builtin_amdgcn_sched_barrier(0);
       // (the first block has no maximum yet.  Lane j < 16 holds the sums of q-rows j and j + 16 in d_new[0]
       // and d_new[1]; a NaN byte of either row makes its own sum NaN whatever the hardware makes of 0 x NaN)
@@ -615,9 +522,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     // phase, measured 2 % slower at D = 128, 7 % with the dense mask)
     if constexpr (EXACT) {   // (the fast path has issued these reads already)
       read_k_frags(sk1);
-#ifndef V_AFTER_QK
       if constexpr (D == 64) read_v_frags(sv);
-#endif
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (D == 128) {
@@ -637,10 +542,6 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     } else {
       qk_mfma();
       __builtin_amdgcn_sched_barrier(0);
-#ifdef V_AFTER_QK
-      read_v_frags(sv);
-      __builtin_amdgcn_sched_barrier(0);
-#endif
     }
     // (fast path: the row sums have been taken above)
 #pragma unroll
@@ -853,7 +754,7 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
                             int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
                             int64_t o_stride_n, float sm_scale, int is_causal, int flags, const int32_t* orders,
                             int n_text, int F, int Hh, int W, void* stream) {
-  PARO_CHECK((flags & ~(PARO_ATTN_EXACT_EXP | PARO_ATTN_PACED | PARO_ATTN_UNPACED)) == 0 &&
+  PARO_CHECK((flags & ~(PARO_ATTN_EXACT_EXP | PARO_ATTN_PACED | PARO_ATTN_UNPACED | PARO_ATTN_TWO_WAVES)) == 0 &&
                  (flags & (PARO_ATTN_PACED | PARO_ATTN_UNPACED)) != (PARO_ATTN_PACED | PARO_ATTN_UNPACED),
              PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
   PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && v_scale && sparse && out, PARO_ERR_RUNTIME,
@@ -901,6 +802,10 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
   hipStream_t st = (hipStream_t)stream;
   const bool dump = s_dump != nullptr;
   const bool exact = (flags & PARO_ATTN_EXACT_EXP) != 0;
+  // D = 64 without lse or score dump: one wave per q-block (attn_sparse_w64.hip), unless the caller asks for the
+  // two-wave kernel or the launch is to be paced (only the two-wave kernel has the paced form)
+  if (D == 64 && lse == nullptr && !dump && (flags & PARO_ATTN_TWO_WAVES) == 0 && !want_pacing(p, D))
+    return launch_attn_w64(p, out_dtype, is_causal != 0, exact, st);
   if (D == 64) {
     if (out_dtype == PARO_DTYPE_F16) return dispatch_attn<64, PARO_DTYPE_F16>(p, is_causal, dump, exact, st);
     return dispatch_attn<64, PARO_DTYPE_BF16>(p, is_causal, dump, exact, st);

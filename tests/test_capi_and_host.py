@@ -11,8 +11,8 @@ import torch
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "paroatten.h")).read()
+def _declared_symbols(header="paroatten.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(paro_[a-z0-9_]+)\s*\(", text)))
 
@@ -30,6 +30,28 @@ def test_library_exports_every_declared_symbol():
     assert lib.paro_build_arch() == b"gfx950"
     raw = ctypes.CDLL(str(L.LIB_PATH))
     assert raw.paro_abi_version() == 1
+
+
+def test_measurement_aids_live_outside_the_product_library():
+    """include/paroatten_diag.h (bench.py --mfma-ceiling / --proxy-ceiling) is a library of its own: every symbol
+    it declares is exported there, none of them by libparoatten_hip.so, and its argument checks answer on the CPU."""
+    import paroatten_amd._lib as L
+    names = _declared_symbols("paroatten_diag.h")
+    assert len(names) >= 7 and all(n.startswith("paro_diag_") for n in names)
+    diag = ctypes.CDLL(str(L.LIB_PATH.parent / "libparoatten_diag.so"))
+    product = ctypes.CDLL(str(L.LIB_PATH))
+    for n in names:
+        assert hasattr(diag, n), f"{n} declared in include/paroatten_diag.h but not exported"
+        assert not hasattr(product, n), f"{n} leaked into the product library"
+        assert n not in L.SIGNATURES
+    assert not any(n.startswith("paro_diag_") for n in _declared_symbols())
+    diag.paro_diag_last_error.restype = ctypes.c_char_p
+    assert diag.paro_diag_attn_proxy(7, None, None, None, 1, 1, 4, None) == -1
+    assert b"level" in diag.paro_diag_last_error()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.c_void_p(ctypes.addressof(buf))
+    assert diag.paro_diag_attn_proxy(0, p, p, p, 1, 1, 70000, None) == -1      # block list entries are 16 bits
+    assert diag.paro_diag_attn_proxy_w64(0, p, p, p, p, 1, 3, 8, None) == -2     # odd iteration count
 
 
 def test_size_queries_need_no_gpu():
@@ -203,3 +225,27 @@ def test_size_limits_are_rejected_without_gpu():
     rc = lib.paro_attn_sparse_fwd(p, p, p, p, p, p, p, p, 0, p, 0, None, None, 1, 1, 1, 64, Nk, D,
                                   64 * D, 64 * D, D, Nk * D, Nk * D, D, 64 * D, 64 * D, D, 0.125, 0, 0, None)
     assert rc == L.PARO_ERR_RUNTIME and b"local data share" in lib.paro_last_error()
+
+
+def test_import_paroattention_resolves_by_itself():
+    """Callers of the reference do `import paroattention` / `from paroattention.cogvideox import ...`
+    (example/pipeline_cogvideox.py:15-16, paroattention/__init__.py:1-5 of the reference): a fresh interpreter
+    finds the same names here without any set-up call."""
+    import subprocess
+    import sys
+    code = (
+        "import paroattention, paroatten_amd\n"
+        "assert paroattention is paroatten_amd\n"
+        "import paroattention.core, paroattention.quant, paroattention.cogvideox, paroattention.wan\n"
+        "import paroattention.prefetch_utils, paroattention.prefetch_wan\n"
+        "import paroattention._qattn_sm80, paroattention._fused, paroattention._rope\n"
+        "from paroattention import paroattn, paroattn_qk_int8_pv_fp16_cuda, PARO_CogVideoXAttnProcessor2_0, "
+        "PARO_WanAttnProcessor2_0\n"
+        "from paroattention.cogvideox import PARO_CogVideoXAttnProcessor2_0 as C\n"
+        "from paroattention.prefetch_utils import TimestepCallback, SparseMaskPrefetchStream\n"
+        "from paroattention.prefetch_wan import TimestepCallback as TW\n"
+        "from paroattention.quant import per_block_int8, per_warp_int8, sub_mean, per_channel_fp8\n"
+        "assert C is PARO_CogVideoXAttnProcessor2_0 and paroattention.core is paroatten_amd.core\n"
+        "print('ok')\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr[-2000:]

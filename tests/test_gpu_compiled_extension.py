@@ -11,7 +11,10 @@ from paroatten_amd import synth
 @pytest.fixture(scope="module")
 def ext():
     import paroatten_amd
-    return paroatten_amd.compiled_extension()
+    try:
+        return paroatten_amd.compiled_extension()
+    except ImportError as e:     # not built, or torch's HIP libraries cannot be loaded in this process
+        pytest.skip(f"compiled extension unavailable: {e} (build it with `python paroatten_amd/build.py`)")
 
 
 def test_extension_imports_and_rejects_cpu_tensors(ext):
@@ -31,9 +34,14 @@ def test_extension_imports_and_rejects_cpu_tensors(ext):
         ext._fused.quant_per_block_int8_cuda(x, o, s)       # neither overload
     import paroatten_amd
     import sys
-    paroatten_amd.install_alias("paroattention_compiled_alias", compiled=True)
-    assert sys.modules["paroattention_compiled_alias._fused"] is ext._fused
-    assert sys.modules["paroattention_compiled_alias.core"] is paroatten_amd.core
+    name = "paroattention_compiled_alias"
+    try:
+        paroatten_amd.install_alias(name, compiled=True)
+        assert sys.modules[f"{name}._fused"] is ext._fused
+        assert sys.modules[f"{name}.core"] is paroatten_amd.core
+    finally:      # leave no alias behind for the rest of the session
+        for mod in [m for m in sys.modules if m == name or m.startswith(name + ".")]:
+            del sys.modules[mod]
 
 
 @pytest.mark.gpu

@@ -64,6 +64,65 @@ def test_rope_is_a_rotation():
     assert torch.allclose(y, yc)
 
 
+def test_rope_cog_table_closed_form():
+    """The CogVideoX rotary TABLE (the pair the reference consumes at cogvideox.py:167-172) in the
+    documented get_3d_rotary_pos_embed convention, checked against closed forms evaluated here in
+    Python floats: a wrong t/h/w split, concatenated instead of interleaved pairs, or an exponent
+    over D instead of over the group's own dimension each fail it."""
+    import math
+
+    D, grid, theta = 64, (13, 30, 45), 10000.0
+    F, Hh, W = grid
+    cos, sin = O.rope_table_cog(D, grid, theta)
+    assert cos.shape == sin.shape == (F * Hh * W, D) and cos.dtype == sin.dtype == torch.float32
+    assert torch.allclose(cos.double() ** 2 + sin.double() ** 2, torch.ones(F * Hh * W, D, dtype=torch.float64), atol=1e-6)
+    c3, s3 = cos.reshape(F, Hh, W, D), sin.reshape(F, Hh, W, D)
+    # channel groups 16 / 24 / 24 (t / h / w = D/4, 3D/8, 3D/8); each depends on ONE grid axis only
+    groups = ((0, 16, 0, F), (16, 40, 1, Hh), (40, 64, 2, W))
+    for lo, hi, axis, _ in groups:
+        for other in ((1, 7, 11), (12, 29, 44), (5, 0, 31)):
+            for pos in (0, 1, 5):
+                a = [other[0], other[1], other[2]]
+                b = [0, 0, 0]
+                a[axis] = b[axis] = pos
+                assert torch.equal(c3[a[0], a[1], a[2], lo:hi], c3[b[0], b[1], b[2], lo:hi])
+                assert torch.equal(s3[a[0], a[1], a[2], lo:hi], s3[b[0], b[1], b[2], lo:hi])
+    # inside a group of dim_g channels: angle[pos, 2i] = angle[pos, 2i+1] = pos * theta^(-2i/dim_g)
+    for lo, hi, axis, length in groups:
+        dim_g = hi - lo
+        for pos in (1, 2, 7, length - 1):
+            idx = [0, 0, 0]
+            idx[axis] = pos
+            for i in (0, 1, 2, dim_g // 2 - 1):
+                ang = pos * theta ** (-2.0 * i / dim_g)
+                for ch in (lo + 2 * i, lo + 2 * i + 1):      # interleaved: the pair shares its frequency
+                    assert float(c3[idx[0], idx[1], idx[2], ch]) == pytest.approx(math.cos(ang), abs=2e-7)
+                    assert float(s3[idx[0], idx[1], idx[2], ch]) == pytest.approx(math.sin(ang), abs=2e-7)
+        # first frequency of each group is theta^0 = 1 rad per position; the second is NOT (rules out a
+        # concatenated [f0, f1, ..., f0, f1, ...] layout, where channel lo + 1 would hold f1's neighbour f0 ... )
+        one = [0, 0, 0]
+        one[axis] = 1
+        assert float(s3[one[0], one[1], one[2], lo]) == pytest.approx(math.sin(1.0), abs=2e-7)
+        assert float(s3[one[0], one[1], one[2], lo + 1]) == pytest.approx(math.sin(1.0), abs=2e-7)
+        assert float(s3[one[0], one[1], one[2], lo + 2]) == pytest.approx(math.sin(theta ** (-2.0 / dim_g)), abs=2e-7)
+        # ... and an exponent over D (64) instead of dim_g would put theta^(-2/64) there
+        assert abs(float(s3[one[0], one[1], one[2], lo + 2]) - math.sin(theta ** (-2.0 / D))) > 1e-2
+    # the last channel of the t group and the first of the h group belong to different axes
+    assert float(s3[1, 0, 0, 16]) == 0.0 and float(s3[0, 1, 0, 15]) == 0.0 and float(s3[0, 1, 0, 16]) == pytest.approx(math.sin(1.0), abs=2e-7)
+    assert float(s3[0, 0, 1, 39]) == 0.0 and float(s3[0, 0, 1, 40]) == pytest.approx(math.sin(1.0), abs=2e-7)
+
+
+def test_rope_cog_table_of_the_package_is_the_oracles():
+    """paroatten_amd.rope.rope_table_cog is independent code (one concatenation, then one
+    repeat_interleave, float64 angles): bit for bit the oracle's table at the CogVideoX-5b grid."""
+    from paroatten_amd.rope import rope_table_cog
+
+    for D, grid in ((64, (13, 30, 45)), (128, (3, 4, 5))):
+        co, so = O.rope_table_cog(D, grid)
+        cp, sp = rope_table_cog(D, grid)
+        assert torch.equal(co, cp) and torch.equal(so, sp)
+
+
 def test_rope_wan_composition_and_split():
     D, grid = 128, (3, 4, 5)
     f = O.rope_table_wan(D, grid)
