@@ -33,6 +33,34 @@ def cosine(a: torch.Tensor, b: torch.Tensor) -> float:
     return float((a @ b) / (a.norm() * b.norm()).clamp_min(1e-300))
 
 
+ATOL = 2e-2          # the benchmark's tolerance on attention outputs (fp16)
+FP8_STEP = 2.0 ** -4   # one e4m3 rounding (3 mantissa bits) at its worst, relative
+
+
+def assert_attention_close(o: torch.Tensor, o_ref: torch.Tensor, a_ref: torch.Tensor, cos: float = 0.999, what: str = "",
+                           frac_one_step: float = 1e-3):
+    """The one tolerance rule for attention outputs at any shape.  `a_ref` is the oracle's attention with |V| in
+    place of V (same weights p): A_ij = sum_j p_ij |v_j|, the scale an output element is built on.  P and V enter
+    the product as e4m3 codes, each up to 2^-4 off in relative terms, so the error of an element is relative to
+    A, not to the element itself (which cancellation can make arbitrarily small):
+        every element:              |o - o_ref| <= ATOL + 2 * 2^-4 * A   (both roundings at their worst: two
+                                                                          comparable keys of opposite sign)
+        all but 1e-3 of them:       |o - o_ref| <= ATOL + 2^-4 * A       (one rounding at its worst; tests whose
+                                    data is built so that a few keys dominate most rows state a larger fraction)
+        cosine(o, o_ref) >= 0.999.
+    At the benchmark shapes, where long rows average V down to |o| ~ 0.05 (A ~ 0.8 / sqrt(n) scale), the A terms
+    are below a few 1e-3 and the rule is the flat atol 2e-2; on short rows and on rows that a few keys dominate
+    (outputs of order 1) it is what FP8 operands can promise."""
+    e = (o.float() - o_ref.float()).abs()
+    a = a_ref.float()
+    worst = float((e - (ATOL + 2 * FP8_STEP * a)).max())
+    assert worst <= 0.0, f"{what}: |o - o_ref| exceeds {ATOL} + 2^-3 * sum p|v| by {worst:.4g} (max abs err {float(e.max()):.4g})"
+    frac = float((e > ATOL + FP8_STEP * a).float().mean())
+    assert frac <= frac_one_step, f"{what}: {frac:.3g} of the elements exceed {ATOL} + 2^-4 * sum p|v|"
+    c = cosine(o, o_ref)
+    assert c >= cos, f"{what}: cosine {c}"
+
+
 def untile_v8(v8: torch.Tensor, B: int, H: int, N: int, D: int) -> torch.Tensor:
     """FP8 V tiles as paro_v_fp8_pack writes them ([B,H,nb][D/32][2][64 lanes][16 bytes]: byte r of
     lane l of piece (dt, mt) = token 64*kb + 32*mt + 8*(r//4) + 4*(l//32) + r%4, channel 32*dt + l%32)

@@ -6,7 +6,7 @@ the FP8 P.V product is specified to; the oracle keeps P and V in 16/32-bit)."""
 import pytest
 import torch
 
-from conftest import cosine
+from conftest import assert_attention_close, cosine
 from oracle import paro_oracle as O
 from paroatten_amd import synth
 
@@ -29,23 +29,23 @@ def _run(dev, B, H, N, D, dtype, density, seed, Hkv=None, causal=False, smooth_k
     km = k.float().mean(dim=2, keepdim=True).to(dtype) if smooth_k else None
     q8, qs, k8, ks = O.per_warp_int8(q, k, km=km, BLKQ=64, WARPQ=32, BLKK=64)
     o_ref, lse_ref = O.sparse_attention(q8, k8, v, qs, ks, mask_b, D ** -0.5, is_causal=causal, out_dtype=dtype)
+    a_ref, _ = O.sparse_attention(q8, k8, v.abs(), qs, ks, mask_b, D ** -0.5, is_causal=causal, out_dtype=torch.float32)
     m_dev = (mask_b if batch_mask else mask).to(dev)
     out = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), m_dev, is_causal=causal,
                                           smooth_k=smooth_k, return_lse=return_lse, exact_exp=exact_exp)
     o, lse = out if return_lse else (out, None)
-    return o.cpu(), (None if lse is None else lse.cpu()), o_ref, lse_ref / O.LOG2E, mask_b
+    return o.cpu(), (None if lse is None else lse.cpu()), (o_ref, a_ref), lse_ref / O.LOG2E, mask_b
 
 
-def _assert_close(o, o_ref, baseline_shape=False):
-    """atol 2e-2 and cosine >= 0.999 at the benchmark shapes.  The FP8 P.V error is relative
-    (about 3.5 % RMS of the output magnitude, measured), so on the reduced shapes below, whose
-    short rows give outputs several times larger than any benchmark shape does, the absolute bound
-    scales with the largest output instead: 8 % of max|o_ref| (never below 2e-2)."""
-    err = (o.float() - o_ref.float()).abs().max().item()
-    c = cosine(o, o_ref)
-    atol = ATOL if baseline_shape else max(ATOL, 0.08 * o_ref.float().abs().max().item())
-    assert err <= atol, f"max abs err {err} > {atol}"
-    assert c >= COS, f"cosine {c}"
+def _assert_close(o, ref, baseline_shape=False):
+    """ref = (o_ref, a_ref) as _run returns them: the one rule of conftest.assert_attention_close
+    (|o - o_ref| <= 2e-2 + 2^-3 * sum_j p_ij |v_j|, all but 1e-3 within 2e-2 + 2^-4 * that, cosine >= 0.999); at a benchmark shape additionally the
+    flat atol 2e-2 the benchmark states."""
+    o_ref, a_ref = ref
+    assert_attention_close(o, o_ref, a_ref, COS)
+    if baseline_shape:
+        err = (o.float() - o_ref.float()).abs().max().item()
+        assert err <= ATOL, f"max abs err {err} > {ATOL}"
 
 
 def test_cfg0_plumbing(dev):
@@ -55,13 +55,13 @@ def test_cfg0_plumbing(dev):
     _assert_close(o, o_ref, baseline_shape=True)
     assert torch.allclose(lse, lse_ref, atol=2e-3, rtol=1e-4)
     for h in range(2):
-        assert cosine(o[:, h], o_ref[:, h]) >= COS
+        assert cosine(o[:, h], o_ref[0][:, h]) >= COS
     for exact in (False, True):
         o2, _, o_ref2, _, _ = _run(dev, 1, 2, 4096, 64, torch.float16, 0.5, seed=0, return_lse=False,
                                    exact_exp=exact)
         _assert_close(o2, o_ref2, baseline_shape=True)
         for h in range(2):
-            assert cosine(o2[:, h], o_ref2[:, h]) >= COS
+            assert cosine(o2[:, h], o_ref2[0][:, h]) >= COS
     assert torch.equal(o2, o)  # exact_exp without lse == the lse instantiation
 
 
@@ -120,9 +120,10 @@ def test_no_smoothing_paths(dev):
     mask = synth.make_block_mask(H, 8, 0.6, seed=22)
     q8, qs, k8, ks = O.per_warp_int8(q, k, BLKQ=64, WARPQ=32, BLKK=64)
     o_ref, _ = O.sparse_attention(q8, k8, v, qs, ks, mask[None], D ** -0.5)
+    a_ref, _ = O.sparse_attention(q8, k8, v.abs(), qs, ks, mask[None], D ** -0.5, out_dtype=torch.float32)
     o = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), smooth_k=False,
                                         smooth_v=False).cpu()
-    _assert_close(o, o_ref)
+    _assert_close(o, (o_ref, a_ref))
 
 
 def test_head_dim_padding(dev):
@@ -133,9 +134,10 @@ def test_head_dim_padding(dev):
     pad = lambda t: torch.nn.functional.pad(t, (0, 128 - D))
     q8, qs, k8, ks = O.per_warp_int8(pad(q), pad(k), BLKQ=64, WARPQ=32, BLKK=64)
     o_ref, _ = O.sparse_attention(q8, k8, pad(v), qs, ks, mask[None], D ** -0.5, out_dtype=torch.bfloat16)
+    a_ref, _ = O.sparse_attention(q8, k8, pad(v).abs(), qs, ks, mask[None], D ** -0.5, out_dtype=torch.float32)
     o = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev)).cpu()
     assert o.shape == (B, H, N, D)
-    _assert_close(o, o_ref[..., :D])
+    _assert_close(o, (o_ref[..., :D], a_ref[..., :D]))
 
 
 @pytest.mark.parametrize("D", [64, 128])
@@ -229,14 +231,13 @@ def test_fast_path_maximum_recovery(dev, D, pattern, causal, density):
     q8, qs, k8, ks = O.per_warp_int8(q, k, BLKQ=64, WARPQ=32, BLKK=64)
     o_ref, _ = O.sparse_attention(q8, k8, v, qs, ks, mask[None], D ** -0.5, is_causal=causal, out_dtype=torch.float32)
     # rows that one or a few keys dominate: the error is FP8's relative rounding error on each product
-    # p*v (at most 2^-4 for V's code and for P's), so the elementwise bound is 0.125 * sum_j p_ij |v_j|
+    # p*v (at most 2^-4 for V's code and for P's), so the elementwise bound is relative to sum_j p_ij |v_j| (conftest.assert_attention_close)
     a_ref, _ = O.sparse_attention(q8, k8, v.abs(), qs, ks, mask[None], D ** -0.5, is_causal=causal,
                                   out_dtype=torch.float32)
 
     def close(a, b):
-        e = (a.float() - b.float()).abs()
-        assert bool((e <= ATOL + 0.125 * a_ref).all()), float((e - 0.125 * a_ref).max())
-        assert cosine(a, b) >= COS, cosine(a, b)
+        # (every row of this case hangs on one or two keys: two roundings coincide on about 1 % of the elements)
+        assert_attention_close(a, b, a_ref, COS, frac_one_step=2e-2)
     # the case does what it is meant to: block maxima climb by more than the headroom many times per row
     s = O.qk_int32(q8, k8)[0, 0].double() * qs[0, 0].double().repeat_interleave(32)[:N, None] \
         * ks[0, 0].double().repeat_interleave(64)[None, :N] * (D ** -0.5) * O.LOG2E
@@ -287,9 +288,7 @@ def test_fast_path_overflow_of_a_single_row(dev, D, row):
     o_exact = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), exact_exp=True, **kw).cpu()
     assert torch.isfinite(o_fast.float()).all()
     for got in (o_fast, o_exact):
-        e = (got.float() - o_ref).abs()
-        assert bool((e <= ATOL + 0.125 * a_ref).all()), float((e - 0.125 * a_ref).max())
-        assert cosine(got, o_ref) >= COS
+        assert_attention_close(got, o_ref, a_ref, COS)
     # the row itself is dominated by the one key: its output is that key's V row to FP8 accuracy
     dom = o_fast[0, 0, qrow].float()
     assert cosine(dom, v[0, 0, key].float()) >= 0.995
@@ -329,7 +328,9 @@ def test_paced_launch_is_bit_identical(dev, D, H, N, monkeypatch):
     h = 3
     o_ref, _ = O.sparse_attention(q8[:, h:h + 1].cpu(), k8[:, h:h + 1].cpu(), v[:, h:h + 1].cpu(), qs[:, h:h + 1].cpu(),
                                   ks[:, h:h + 1].cpu(), mask[None, h:h + 1].cpu(), D ** -0.5, out_dtype=torch.float32)
-    _assert_close(outs[1][0][:, h:h + 1].cpu(), o_ref, baseline_shape=True)
+    a_ref, _ = O.sparse_attention(q8[:, h:h + 1].cpu(), k8[:, h:h + 1].cpu(), v[:, h:h + 1].cpu().abs(), qs[:, h:h + 1].cpu(),
+                                  ks[:, h:h + 1].cpu(), mask[None, h:h + 1].cpu(), D ** -0.5, out_dtype=torch.float32)
+    _assert_close(outs[1][0][:, h:h + 1].cpu(), (o_ref, a_ref), baseline_shape=True)
     # the fast-exponential instantiation and the folded inverse permutation go through the same launch code
     a = torch.empty_like(q)
     b = torch.empty_like(q)
