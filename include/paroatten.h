@@ -246,6 +246,25 @@ int paro_rope_k_mean(const void* k, int dtype, const float* cos, const float* si
                      int B, int H, int N, int D, int n_text, int F, int Hh, int W,
                      int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
                      int64_t mean_stride_b, int64_t mean_stride_h, void* stream);
+/* paro_rope_k_mean followed by paro_rope_permute_quant_fwd with that mean, as one call: what a caller that
+ * smooths K does per layer (the reference's quantiser takes `km = k.mean(dim=seq)`, paroattention/quant.py:105-180,
+ * 174-176).  k_mean is an OUTPUT here ([B,H,D] in the input dtype through the mean strides), filled before it
+ * is used; the results are bit-identical to the two calls.  The K sums and the V statistics, both plain
+ * streaming passes, share one launch and their second steps another (four launches instead of six).
+ * workspace: paro_prep_smooth_workspace_bytes() bytes (the K and V partial results are alive together). */
+int64_t paro_prep_smooth_workspace_bytes(int B, int H, int N, int D);
+int paro_rope_k_mean_permute_quant_fwd(const void* q, const void* k, const void* v, int dtype,
+                                       const float* cos, const float* sin, const int32_t* orders,
+                                       void* k_mean,
+                                       int8_t* q8, float* q_scale, int8_t* k8, float* k_scale,
+                                       uint8_t* v8, float* v_scale, float* v_mean,
+                                       void* workspace, int64_t workspace_bytes,
+                                       int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                                       int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                                       int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                       int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                                       int64_t mean_stride_b, int64_t mean_stride_h,
+                                       int smooth_v, void* stream);
 
 /* paro_rope_k_mean for callers that can neither allocate device memory nor bring a workspace (code under
  * HIP graph capture, serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the

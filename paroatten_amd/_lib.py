@@ -60,6 +60,10 @@ SIGNATURES = {
     "paro_rope_permute_quant_fwd": (c_int, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L,
                                             _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _L,
                                             _L, _L, _I, _P]),
+    "paro_prep_smooth_workspace_bytes": (c_int64, [_I, _I, _I, _I]),
+    "paro_rope_k_mean_permute_quant_fwd": (c_int, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L,
+                                                   _I, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _L,
+                                                   _L, _L, _I, _P]),
     "paro_rope_k_mean": (c_int, [_P, _I, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _I,
                                  _L, _L, _L, _L, _L, _P]),
     "paro_rope_k_mean_static": (c_int, [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I,

@@ -146,8 +146,9 @@ class _ParoProcessorBase:
             # keys that must not be rotated: rotate the queries separately, then prepare without tables
             query, _, _ = PM.rope_permute(query, None, None, torch.zeros_like(orders), grid, n_text, cos, sin)
             cos = sin = None
-        km = PM.rope_k_mean(key, grid, n_text, cos, sin) if self.smooth_k else None
-        return PM.rope_permute_quant(query, key, value, orders, grid, n_text, cos, sin, km=km)
+        # (smoothing: the mean of the rotated K is taken inside the same call)
+        return PM.rope_permute_quant(query, key, value, orders, grid, n_text, cos, sin,
+                                     km="mean" if self.smooth_k else None)
 
     def _sparse_attention(self, ops, out, sm_scale, orders, grid, n_text):
         """Block-sparse attention on the prepared operands; the inverse permutation (permute_attn_out)

@@ -18,7 +18,8 @@
 // Reference for the arithmetic: the RoPE + permute_qk sequence of the processors
 // (paroattention/cogvideox.py:167-186), QuantInt8Kernel (csrc/fused/fused.cu:64-198) and
 // MeanScaleKernel (csrc/fused/fused.cu:316-427).
-#include "paro_device.hpp"
+#include "stats_device.hpp"
+#include <stdlib.h>
 #include <mutex>
 
 namespace paro {
@@ -339,109 +340,57 @@ __global__ void __launch_bounds__(256) rope_permute_quant_kernel(const PrepParam
   wait_vm<0>();
 }
 
-// K mean over tokens AFTER the rotation (the permutation does not change a mean): partial sums per
-// K_CHUNK-token chunk, then one workgroup per (batch, head) adds them in a fixed order.  A thread keeps
-// the table entries of its token piece while it walks over a group of (batch, head) pairs.
-constexpr int KM_GROUP = 4;   // measured: 4 beats 8 (too few workgroups at 40 heads) and 2 (tables re-read twice as often)
-template <int DT, int D>
+// K mean over tokens AFTER the rotation (the permutation does not change a mean) and the V statistics: the bodies
+// live in stats_device.hpp.  Alone (paro_rope_k_mean), or both in ONE launch when the preparation smooths K
+// itself: a workgroup takes a K chunk of a head group or a V chunk of a head, and one more launch finishes both.
+template <int DT, int D, int KB>
 __global__ void __launch_bounds__(256) rope_k_sum_kernel(const unsigned short* __restrict__ k,
                                                          const float* __restrict__ cos_t,
                                                          const float* __restrict__ sin_t,
                                                          float* __restrict__ partial, int BH, int H, int N,
                                                          int n_text, int n_chunks, int64_t ks_b, int64_t ks_h,
                                                          int64_t ks_n) {
-  constexpr int LPR = D / 8;
-  constexpr int ROWS = 256 / LPR;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  // Workgroup ids are dealt round-robin to the 8 XCDs: XCD x takes the token chunks 8*i + x, and for each of
-  // them all head groups one after the other, so that a chunk of the rotary tables (twice the bytes of the
-  // K rows of one head) crosses the fabric once per launch and is served to the other head groups by that
-  // XCD's L2.
-  const int n_hg = (BH + KM_GROUP - 1) / KM_GROUP;
-  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-  const int chunk = (j / n_hg) * 8 + xcd;
-  if (chunk >= n_chunks) return;
-  const int bh0 = (j % n_hg) * KM_GROUP;
-  const int col = (t % LPR) * 8;
-  float s[KM_GROUP][8];
-#pragma unroll
-  for (int g = 0; g < KM_GROUP; g++)
-#pragma unroll
-    for (int j = 0; j < 8; j++) s[g][j] = 0.f;
-  for (int r = t / LPR; r < K_CHUNK; r += ROWS) {
-    const int tok = chunk * K_CHUNK + r;
-    if (tok >= N) break;
-    const bool rot = cos_t != nullptr && tok >= n_text;
-    float cs[8], sn[8];
-    if (rot) {
-      const int64_t o = (int64_t)(tok - n_text) * D + col;
-      const v4f c0 = *reinterpret_cast<const v4f*>(cos_t + o), c1 = *reinterpret_cast<const v4f*>(cos_t + o + 4);
-      const v4f s0 = *reinterpret_cast<const v4f*>(sin_t + o), s1 = *reinterpret_cast<const v4f*>(sin_t + o + 4);
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        cs[j] = c0[j]; cs[4 + j] = c1[j];
-        sn[j] = s0[j]; sn[4 + j] = s1[j];
-      }
-    }
-#pragma unroll
-    for (int g = 0; g < KM_GROUP; g++) {
-      const int bh = bh0 + g;
-      if (bh < BH) {
-        const int b = bh / H, h = bh - b * H;
-        // ordinary load: K was just written by the projection and is read again by the preparation
-        // pass, so it should stay in the last-level cache
-        v4i raw = *reinterpret_cast<const v4i*>(k + b * ks_b + h * ks_h + (int64_t)tok * ks_n + col);
-        if (rot) raw = rotate8<DT>(raw, cs, sn);
-#pragma unroll
-        for (int j = 0; j < 8; j++) s[g][j] += elem16_to_f32<DT>(raw, j);
-      }
-    }
-  }
-  __shared__ float red[4][KM_GROUP][D];
-#pragma unroll
-  for (int g = 0; g < KM_GROUP; g++) {
-    // lanes that share a column sit LPR apart
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      float a, b;
-      if constexpr (LPR == 8) s[g][j] += row_dpp<0x128>(s[g][j]);
-      with_lane_xor16(s[g][j], a, b);
-      s[g][j] = a + b;
-      with_lane_xor32(s[g][j], a, b);
-      s[g][j] = a + b;
-    }
-    if (lane < LPR) {
-#pragma unroll
-      for (int j = 0; j < 8; j++) red[wave][g][col + j] = s[g][j];
-    }
-  }
-  __syncthreads();
-  for (int i = t; i < KM_GROUP * D; i += 256) {
-    const int g = i / D, ch = i % D;
-    if (bh0 + g < BH)
-      partial[((int64_t)(bh0 + g) * n_chunks + chunk) * D + ch] =
-          (red[0][g][ch] + red[1][g][ch]) + (red[2][g][ch] + red[3][g][ch]);
-  }
+  rope_k_sum_body<DT, D, KB>(k, cos_t, sin_t, partial, BH, H, N, n_text, n_chunks, ks_b, ks_h, ks_n, blockIdx.x);
 }
 
 template <int DT, int D>
 __global__ void __launch_bounds__(1024) k_mean_finalize_kernel(const float* __restrict__ partial,
                                                                unsigned short* __restrict__ k_mean, int N,
                                                                int n_chunks, int64_t ms_b, int64_t ms_h, int H) {
-  constexpr int SL = 1024 / D;
-  __shared__ float red[SL][D];
-  const int ch = threadIdx.x % D, sl = threadIdx.x / D;
-  const int64_t bh = blockIdx.x;
-  const float* p = partial + bh * n_chunks * D;
-  float s = 0.f;
-  for (int c = sl; c < n_chunks; c += SL) s += p[c * D + ch];
-  red[sl][ch] = s;
-  __syncthreads();
-  if (sl == 0) {
-    for (int i = 1; i < SL; i++) s += red[i][ch];
-    const int b = (int)(bh / H), h = (int)(bh % H);
-    k_mean[b * ms_b + h * ms_h + ch] = (unsigned short)(pack2_from_f32<DT>(s / (float)N, 0.f) & 0xffffu);
+  k_mean_finalize_body<DT, D>(partial, k_mean, N, n_chunks, ms_b, ms_h, H, blockIdx.x);
+}
+
+// workgroups of the K sums: XCD x takes the chunks 8*i + x, and for each of them all head groups
+static inline int k_sum_blocks(int n_chunks, int BH) { return ceil_div(n_chunks, 8) * 8 * ceil_div(BH, KM_GROUP); }
+
+struct KvStatsParams {
+  const unsigned short* k; const unsigned short* v;
+  const float* cos_t; const float* sin_t;
+  float* k_partial; float* v_partial;
+  unsigned short* k_mean; float* v_scale; float* v_mean;
+  int B, H, N, n_text, k_chunks, v_chunks, k_blocks, smooth_v;
+  int64_t ks_b, ks_h, ks_n, vs_b, vs_h, vs_n, ms_b, ms_h;
+};
+
+template <int DT, int D, int KB>
+__global__ void __launch_bounds__(256) kv_stats_kernel(const KvStatsParams p) {
+  if ((int)blockIdx.x < p.k_blocks) {
+    rope_k_sum_body<DT, D, KB>(p.k, p.cos_t, p.sin_t, p.k_partial, p.B * p.H, p.H, p.N, p.n_text, p.k_chunks, p.ks_b,
+                               p.ks_h, p.ks_n, blockIdx.x);
+  } else {
+    const int i = blockIdx.x - p.k_blocks;
+    const int chunk = i % p.v_chunks, bh = i / p.v_chunks;
+    v_stats_body<DT, D>(p.v, p.v_partial, p.N, p.v_chunks, p.vs_b, p.vs_h, p.vs_n, chunk, bh % p.H, bh / p.H, p.H);
   }
+}
+
+template <int DT, int D>
+__global__ void __launch_bounds__(1024) kv_finalize_kernel(const KvStatsParams p) {
+  const int BH = p.B * p.H;
+  if ((int)blockIdx.x < BH)
+    k_mean_finalize_body<DT, D>(p.k_partial, p.k_mean, p.N, p.k_chunks, p.ms_b, p.ms_h, p.H, blockIdx.x);
+  else
+    v_finalize_body<D>(p.v_partial, p.v_scale, p.v_mean, p.N, p.v_chunks, p.smooth_v, (int64_t)blockIdx.x - BH);
 }
 
 template <int DT, int D>
@@ -496,9 +445,10 @@ extern "C" int paro_rope_k_mean(const void* k, int dtype, const float* cos, cons
              "paro_rope_k_mean: workspace of %lld bytes is too small", (long long)workspace_bytes);
   hipStream_t st = (hipStream_t)stream;
   float* partial = (float*)workspace;
+  // tokens per thread whose loads are requested together: 2 at D = 64, 1 at D = 128 (measured)
 #define PARO_KM(DTV, DV)                                                                                        \
   do {                                                                                                          \
-    hipLaunchKernelGGL((rope_k_sum_kernel<DTV, DV>), dim3(ceil_div(n_chunks, 8) * 8 * ceil_div(B * H, KM_GROUP)), dim3(256), 0, \
+    hipLaunchKernelGGL((rope_k_sum_kernel<DTV, DV, (DV == 64 ? 2 : 1)>), dim3(k_sum_blocks(n_chunks, B * H)), dim3(256), 0, \
                        st, (const unsigned short*)k, cos, sin, partial, B * H, H, N, n_text, n_chunks,          \
                        k_stride_b, k_stride_h, k_stride_n);                                                     \
     hipLaunchKernelGGL((k_mean_finalize_kernel<DTV, DV>), dim3(B * H), dim3(1024), 0, st, (const float*)partial, \
@@ -534,7 +484,10 @@ extern "C" int paro_rope_k_mean_static(const void* k, int dtype, const float* co
                           k_stride_b, k_stride_h, k_stride_n, mean_stride_b, mean_stride_h, stream);
 }
 
-extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const void* v, int dtype, const float* cos,
+namespace paro {
+// compute_k_mean: k_mean is an output (the mean of the rotated K, as paro_rope_k_mean gives it) that this call
+// fills before it uses it; the K sums and the V statistics then share one launch, and so do their second steps.
+static int prep_impl(bool compute_k_mean, const void* q, const void* k, const void* v, int dtype, const float* cos,
                                            const float* sin, const int32_t* orders, const void* k_mean,
                                            int8_t* q8, float* q_scale, int8_t* k8, float* k_scale, uint8_t* v8,
                                            float* v_scale, float* v_mean, void* workspace, int64_t workspace_bytes,
@@ -544,7 +497,6 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
                                            int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
                                            int64_t mean_stride_b, int64_t mean_stride_h, int smooth_v,
                                            void* stream) {
-  using namespace paro;
   if (int rc = check_prep("paro_rope_permute_quant_fwd", dtype, B, H, N, D, n_text, F, Hh, W, q_stride_b,
                           q_stride_h, q_stride_n))
     return rc;
@@ -562,7 +514,10 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
                "paro_rope_permute_quant_fwd: tensors must be 16-byte aligned");
   PARO_CHECK(!k_mean || (mean_stride_b % 8 == 0 && mean_stride_h % 8 == 0), PARO_ERR_RUNTIME,
              "Tensor mean must be 16-byte aligned with strides that are multiples of 8");
-  PARO_CHECK(workspace_bytes >= paro_prep_workspace_bytes(B, H, N, D) && ((uintptr_t)workspace % 16) == 0,
+  PARO_CHECK(!compute_k_mean || k_mean, PARO_ERR_RUNTIME, "paro_rope_k_mean_permute_quant_fwd: null k_mean");
+  PARO_CHECK(workspace_bytes >= (compute_k_mean ? paro_prep_smooth_workspace_bytes(B, H, N, D)
+                                                : paro_prep_workspace_bytes(B, H, N, D)) &&
+                 ((uintptr_t)workspace % 16) == 0,
              PARO_ERR_RUNTIME, "paro_rope_permute_quant_fwd: workspace of %lld bytes is too small or misaligned",
              (long long)workspace_bytes);
   // one (batch, head) slice of each input and of q8 / k8 is addressed through 32-bit buffer offsets
@@ -573,9 +528,34 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
              PARO_ERR_RUNTIME, "paro_rope_permute_quant_fwd: one head of q, k or v spans 2 GiB or more");
   hipStream_t st = (hipStream_t)stream;
   // V statistics do not depend on the token order: taken on the unpermuted tensor
-  if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, (float*)workspace, B, H, N, D, v_stride_b, v_stride_h,
-                           v_stride_n, smooth_v, st))
-    return rc;
+  if (!compute_k_mean) {
+    if (int rc = v_fp8_stats(v, dtype, v_scale, v_mean, (float*)workspace, B, H, N, D, v_stride_b, v_stride_h,
+                             v_stride_n, smooth_v, st))
+      return rc;
+  } else {
+    KvStatsParams sp;
+    sp.k = (const unsigned short*)k; sp.v = (const unsigned short*)v; sp.cos_t = cos; sp.sin_t = sin;
+    sp.v_partial = (float*)workspace;
+    sp.k_partial = (float*)workspace + paro_v_fp8_partial_floats(B, H, N, D);   // behind the V partials
+    sp.k_mean = (unsigned short*)k_mean; sp.v_scale = v_scale; sp.v_mean = v_mean;
+    sp.B = B; sp.H = H; sp.N = N; sp.n_text = n_text; sp.k_chunks = ceil_div(N, K_CHUNK); sp.v_chunks = ceil_div(N, V_CHUNK);
+    sp.k_blocks = k_sum_blocks(sp.k_chunks, B * H); sp.smooth_v = smooth_v;
+    sp.ks_b = k_stride_b; sp.ks_h = k_stride_h; sp.ks_n = k_stride_n;
+    sp.vs_b = v_stride_b; sp.vs_h = v_stride_h; sp.vs_n = v_stride_n; sp.ms_b = mean_stride_b; sp.ms_h = mean_stride_h;
+    const int n_blocks = sp.k_blocks + sp.v_chunks * B * H;
+#define PARO_KV(DTV, DV)                                                                                          \
+  do {                                                                                                            \
+    hipLaunchKernelGGL((kv_stats_kernel<DTV, DV, (DV == 64 ? 2 : 1)>), dim3(n_blocks), dim3(256), 0, st, sp);      \
+    hipLaunchKernelGGL((kv_finalize_kernel<DTV, DV>), dim3(2 * B * H), dim3(1024), 0, st, sp);                    \
+  } while (0)
+    if (dtype == PARO_DTYPE_F16) {
+      if (D == 64) PARO_KV(PARO_DTYPE_F16, 64); else PARO_KV(PARO_DTYPE_F16, 128);
+    } else {
+      if (D == 64) PARO_KV(PARO_DTYPE_BF16, 64); else PARO_KV(PARO_DTYPE_BF16, 128);
+    }
+#undef PARO_KV
+    PARO_HIP(hipGetLastError());
+  }
   const int nb = ceil_div(N, 64);
   // every order gets `head_split` workgroups per block, each walking over its share of the (batch,
   // head) pairs with that order: enough workgroups to fill the chip, few enough that the table rows a
@@ -606,4 +586,42 @@ extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const v
   PARO_HIP(hipGetLastError());
   if (p.v_resid) return v_fp8_add_residual(p.v_resid, v_scale, v_mean, B, H, N, D, st);
   return PARO_OK;
+}
+}  // namespace paro
+
+extern "C" int64_t paro_prep_smooth_workspace_bytes(int B, int H, int N, int D) {
+  // the V partials and, behind them, the K partial sums: both are alive at the same time
+  return (paro_v_fp8_partial_floats(B, H, N, D) + (int64_t)B * H * paro::ceil_div(N, paro::K_CHUNK) * D) * 4;
+}
+
+extern "C" int paro_rope_permute_quant_fwd(const void* q, const void* k, const void* v, int dtype, const float* cos,
+                                           const float* sin, const int32_t* orders, const void* k_mean,
+                                           int8_t* q8, float* q_scale, int8_t* k8, float* k_scale, uint8_t* v8,
+                                           float* v_scale, float* v_mean, void* workspace, int64_t workspace_bytes,
+                                           int B, int H, int N, int D, int n_text, int F, int Hh, int W,
+                                           int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_n,
+                                           int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_n,
+                                           int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
+                                           int64_t mean_stride_b, int64_t mean_stride_h, int smooth_v,
+                                           void* stream) {
+  return paro::prep_impl(false, q, k, v, dtype, cos, sin, orders, k_mean, q8, q_scale, k8, k_scale, v8, v_scale, v_mean,
+                         workspace, workspace_bytes, B, H, N, D, n_text, F, Hh, W, q_stride_b, q_stride_h, q_stride_n,
+                         k_stride_b, k_stride_h, k_stride_n, v_stride_b, v_stride_h, v_stride_n, mean_stride_b,
+                         mean_stride_h, smooth_v, stream);
+}
+
+extern "C" int paro_rope_k_mean_permute_quant_fwd(const void* q, const void* k, const void* v, int dtype,
+                                                  const float* cos, const float* sin, const int32_t* orders,
+                                                  void* k_mean, int8_t* q8, float* q_scale, int8_t* k8,
+                                                  float* k_scale, uint8_t* v8, float* v_scale, float* v_mean,
+                                                  void* workspace, int64_t workspace_bytes, int B, int H, int N,
+                                                  int D, int n_text, int F, int Hh, int W, int64_t q_stride_b,
+                                                  int64_t q_stride_h, int64_t q_stride_n, int64_t k_stride_b,
+                                                  int64_t k_stride_h, int64_t k_stride_n, int64_t v_stride_b,
+                                                  int64_t v_stride_h, int64_t v_stride_n, int64_t mean_stride_b,
+                                                  int64_t mean_stride_h, int smooth_v, void* stream) {
+  return paro::prep_impl(true, q, k, v, dtype, cos, sin, orders, k_mean, q8, q_scale, k8, k_scale, v8, v_scale, v_mean,
+                         workspace, workspace_bytes, B, H, N, D, n_text, F, Hh, W, q_stride_b, q_stride_h, q_stride_n,
+                         k_stride_b, k_stride_h, k_stride_n, v_stride_b, v_stride_h, v_stride_n, mean_stride_b,
+                         mean_stride_h, smooth_v, stream);
 }

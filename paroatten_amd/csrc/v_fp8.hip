@@ -17,7 +17,7 @@
 // monotonic, so no second reduction pass is needed.
 // Arithmetic follows MeanScaleKernel of the reference (csrc/fused/fused.cu:316-427) except that the
 // mean divides by the true token count.
-#include "paro_device.hpp"
+#include "stats_device.hpp"
 
 namespace paro {
 
@@ -25,120 +25,14 @@ template <int DT, int D>
 __global__ void __launch_bounds__(256) v_stats_kernel(const unsigned short* __restrict__ v,
                                                       float* __restrict__ partial, int N, int n_chunks,
                                                       int64_t vs_b, int64_t vs_h, int64_t vs_n) {
-  constexpr int LPR = D / 8;
-  constexpr int ROWS = 256 / LPR;
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int col = (t % LPR) * 8;
-  const unsigned short* vb = v + b * vs_b + h * vs_h + col;
-  float s[8], mn[8], mx[8];
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    s[j] = 0.f;
-    mn[j] = INFINITY;
-    mx[j] = -INFINITY;
-  }
-  auto take = [&](const v4i raw) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const float f = elem16_to_f32<DT>(raw, j);
-      s[j] += f;
-      mn[j] = fminf(mn[j], f);
-      mx[j] = fmaxf(mx[j], f);
-    }
-  };
-  const int tok0 = chunk * V_CHUNK + t / LPR;
-  if (chunk * V_CHUNK + V_CHUNK <= N) {
-    // full chunk (uniform): batches of VS_BATCH independent loads, then the arithmetic
-    constexpr int VS_BATCH = 8;
-    for (int r = 0; r < V_CHUNK; r += ROWS * VS_BATCH) {
-      v4i raw[VS_BATCH];
-#pragma unroll
-      for (int u = 0; u < VS_BATCH; u++)
-        // (non-temporal: measured 3-5 us faster per launch of the entry point and of the per-layer sequence
-        // than ordinary loads, although the packing pass reads the same tensor right afterwards)
-        raw[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(vb + (int64_t)(tok0 + r + u * ROWS) * vs_n));
-#pragma unroll
-      for (int u = 0; u < VS_BATCH; u++) take(raw[u]);
-    }
-  } else {
-    for (int r = 0; r < V_CHUNK; r += ROWS) {
-      const int tok = tok0 + r;
-      if (tok < N) take(*reinterpret_cast<const v4i*>(vb + (int64_t)tok * vs_n));
-    }
-  }
-  // lanes that share a column sit LPR apart: 8 lanes round the row (D = 64 only), then lane ^ 16, ^ 32
-#pragma unroll
-  for (int j = 0; j < 8; j++) {
-    float a, b;
-    if constexpr (LPR == 8) {
-      s[j] += row_dpp<0x128>(s[j]);
-      mn[j] = fminf(mn[j], row_dpp<0x128>(mn[j]));
-      mx[j] = fmaxf(mx[j], row_dpp<0x128>(mx[j]));
-    }
-    with_lane_xor16(s[j], a, b);  s[j] = a + b;
-    with_lane_xor16(mn[j], a, b); mn[j] = fminf(a, b);
-    with_lane_xor16(mx[j], a, b); mx[j] = fmaxf(a, b);
-    with_lane_xor32(s[j], a, b);  s[j] = a + b;
-    with_lane_xor32(mn[j], a, b); mn[j] = fminf(a, b);
-    with_lane_xor32(mx[j], a, b); mx[j] = fmaxf(a, b);
-  }
-  __shared__ float red[4][3][D];
-  if (lane < LPR) {
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      red[wave][0][col + j] = s[j];
-      red[wave][1][col + j] = mn[j];
-      red[wave][2][col + j] = mx[j];
-    }
-  }
-  __syncthreads();
-  if (t < D) {
-    const float ss = (red[0][0][t] + red[1][0][t]) + (red[2][0][t] + red[3][0][t]);
-    const float mm = fminf(fminf(red[0][1][t], red[1][1][t]), fminf(red[2][1][t], red[3][1][t]));
-    const float xx = fmaxf(fmaxf(red[0][2][t], red[1][2][t]), fmaxf(red[2][2][t], red[3][2][t]));
-    float* p = partial + (((int64_t)(b * gridDim.y + h) * n_chunks + chunk) * 3) * D;
-    p[t] = ss;
-    p[D + t] = mm;
-    p[2 * D + t] = xx;
-  }
+  v_stats_body<DT, D>(v, partial, N, n_chunks, vs_b, vs_h, vs_n, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.y);
 }
 
 template <int D>
 __global__ void __launch_bounds__(1024) v_finalize_kernel(float* partial, float* __restrict__ v_scale,
                                                           float* __restrict__ v_mean, int N, int n_chunks,
                                                           int smooth) {
-  // 1024 / D slices of the chunk range per channel, combined through LDS in a fixed order
-  constexpr int SL = 1024 / D;
-  __shared__ float red[3][SL][D];
-  const int ch = threadIdx.x % D, sl = threadIdx.x / D;
-  const int64_t bh = blockIdx.x;
-  const float* p = partial + bh * n_chunks * 3 * D;
-  float s = 0.f, mn = INFINITY, mx = -INFINITY;
-  for (int c = sl; c < n_chunks; c += SL) {
-    s += p[(c * 3 + 0) * D + ch];
-    mn = fminf(mn, p[(c * 3 + 1) * D + ch]);
-    mx = fmaxf(mx, p[(c * 3 + 2) * D + ch]);
-  }
-  red[0][sl][ch] = s;
-  red[1][sl][ch] = mn;
-  red[2][sl][ch] = mx;
-  __syncthreads();
-  if (sl == 0) {
-    for (int i = 1; i < SL; i++) {
-      s += red[0][i][ch];
-      mn = fminf(mn, red[1][i][ch]);
-      mx = fmaxf(mx, red[2][i][ch]);
-    }
-    const float mean = smooth ? s / (float)N : 0.f;
-    const float amax = fmaxf(mx - mean, mean - mn);
-    v_scale[bh * D + ch] = amax / 448.0f;
-    if (v_mean) v_mean[bh * D + ch] = mean;
-    // every thread of this workgroup has read its partials before the barrier above: the head of the
-    // region is free to carry the reciprocal, and behind it the mean, to the pack kernel
-    partial[v_recp_offset(bh, n_chunks, D) + ch] = amax > 0.f ? 448.0f / amax : 0.f;
-    partial[v_recp_offset(bh, n_chunks, D) + D + ch] = mean;
-  }
+  v_finalize_body<D>(partial, v_scale, v_mean, N, n_chunks, smooth, blockIdx.x);
 }
 
 template <int DT, int D>

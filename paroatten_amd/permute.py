@@ -84,6 +84,7 @@ class PreparedOperands(NamedTuple):
     v8: torch.Tensor
     v_scale: torch.Tensor
     v_mean: Optional[torch.Tensor]
+    k_mean: Optional[torch.Tensor] = None   # the rotated K mean, when the call computed it itself (km="mean")
 
 
 def _tables_ok(cos, sin, n_img, D):
@@ -114,12 +115,14 @@ def rope_k_mean(k: torch.Tensor, grid: Sequence[int], n_text: int, cos: Optional
 
 def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders: torch.Tensor,
                        grid: Sequence[int], n_text: int, cos: Optional[torch.Tensor] = None,
-                       sin: Optional[torch.Tensor] = None, km: Optional[torch.Tensor] = None,
+                       sin: Optional[torch.Tensor] = None, km=None,
                        smooth_v: bool = True) -> PreparedOperands:
     """rope_permute + per_warp_int8(BLKQ=64, WARPQ=32, BLKK=64, km) + per_channel_fp8 in one pass, with
     bit-identical INT8 results and without the permuted 16-bit tensors ever being written.  q, k, v:
-    [B,H,N,D] views, each with its own strides (e.g. the transposed token-major projections); km: None or
-    [B,H,1,D] in the input dtype (see rope_k_mean)."""
+    [B,H,N,D] views, each with its own strides (e.g. the transposed token-major projections); km: None,
+    [B,H,1,D] in the input dtype (see rope_k_mean), or the string "mean": the mean of the rotated K is taken
+    inside the same call (its pass over K shares a launch with the V statistics) and returned as the `k_mean`
+    field of the result."""
     _check_hnd(q, "query")
     B, H, N, D = q.shape
     for t, n in ((k, "key"), (v, "value")):
@@ -130,6 +133,11 @@ def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders
     F, Hh, W = (int(x) for x in grid)
     _tables_ok(cos, sin, F * Hh * W, D)
     ms_b = ms_h = 0
+    compute_km = isinstance(km, str)
+    if compute_km:
+        if km != "mean":
+            raise ValueError("km must be None, a tensor, or the string 'mean'")
+        km = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
     if km is not None:
         _lib.require_gpu(km, "km")
         if km.dtype != q.dtype or tuple(km.shape) != (B, H, 1, D) or km.stride(-1) != 1:
@@ -145,13 +153,15 @@ def rope_permute_quant(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, orders
     v8 = torch.empty(int(lib.paro_v_fp8_bytes(B, H, N, D)), dtype=torch.uint8, device=dev)
     v_scale = torch.empty((B, H, D), dtype=torch.float32, device=dev)
     v_mean = torch.empty((B, H, D), dtype=torch.float32, device=dev)
-    ws = torch.empty(int(lib.paro_prep_workspace_bytes(B, H, N, D)), dtype=torch.uint8, device=dev)
-    _lib.on(q).paro_rope_permute_quant_fwd(
+    ws_bytes = lib.paro_prep_smooth_workspace_bytes(B, H, N, D) if compute_km else lib.paro_prep_workspace_bytes(B, H, N, D)
+    ws = torch.empty(int(ws_bytes), dtype=torch.uint8, device=dev)
+    entry = _lib.on(q).paro_rope_k_mean_permute_quant_fwd if compute_km else _lib.on(q).paro_rope_permute_quant_fwd
+    entry(
         ptr(q), ptr(k), ptr(v), _lib.DTYPE_CODE[q.dtype], ptr(cos), ptr(sin), ptr(orders), ptr(km),
         ptr(q8), ptr(q_scale), ptr(k8), ptr(k_scale), ptr(v8), ptr(v_scale), ptr(v_mean), ptr(ws), ws.numel(),
         B, H, N, D, int(n_text), F, Hh, W, q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1),
         k.stride(2), v.stride(0), v.stride(1), v.stride(2), ms_b, ms_h, 1 if smooth_v else 0, stream_of(q))
-    return PreparedOperands(q8, q_scale, k8, k_scale, v8, v_scale, v_mean if smooth_v else None)
+    return PreparedOperands(q8, q_scale, k8, k_scale, v8, v_scale, v_mean if smooth_v else None, km if compute_km else None)
 
 
 def permute_inverse(o: torch.Tensor, orders: torch.Tensor, grid: Sequence[int], n_text: int,

@@ -211,3 +211,29 @@ def test_attention_with_folded_inverse_permutation(dev, D, grid, n_text, dtype):
     with pytest.raises(RuntimeError):
         qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, plain, ops.q_scale, ops.k_scale,
                                     D ** -0.5, mask, unpermute=(orders, (grid[0], grid[1], grid[2] + 1), n_text))
+
+
+@pytest.mark.parametrize("B,H,D,grid,n_text,dtype,rope_kind", [
+    (2, 5, 64, (3, 10, 11), 35, torch.float16, "cog"),      # a text prefix inside the first chunk, ragged last chunk
+    (1, 6, 128, (4, 9, 31), 0, torch.bfloat16, "wan"),
+    (1, 3, 64, (2, 8, 8), 0, torch.bfloat16, None),         # no rotation, fewer heads than a head group
+])
+def test_k_mean_inside_the_preparation_call(dev, B, H, D, grid, n_text, dtype, rope_kind):
+    """km="mean" (paro_rope_k_mean_permute_quant_fwd: the K sums and the V statistics in one launch, their
+    second steps in another) against rope_k_mean followed by rope_permute_quant with that mean: every output
+    bit for bit, the mean included."""
+    from paroatten_amd import permute as PM
+    q, k, v, plan, cos, sin, N = _case(dev, B, H, D, grid, n_text, dtype, 41, rope_kind)
+    q, k, v = q.to(dev), k.to(dev), v.to(dev)
+    k = k + 2.0     # a mean worth subtracting
+    cos, sin = (None, None) if cos is None else (cos.to(dev), sin.to(dev))
+    orders = PM.head_orders(plan, 0, dev)
+    km = PM.rope_k_mean(k, grid, n_text, cos, sin)
+    two = PM.rope_permute_quant(q, k, v, orders, grid, n_text, cos, sin, km=km)
+    one = PM.rope_permute_quant(q, k, v, orders, grid, n_text, cos, sin, km="mean")
+    assert two.k_mean is None and one.k_mean is not None
+    assert torch.equal(one.k_mean.view(torch.int16), km.view(torch.int16))
+    for name in ("q8", "q_scale", "k8", "k_scale", "v8", "v_scale", "v_mean"):
+        a, b = getattr(one, name), getattr(two, name)
+        assert torch.equal(a.view(torch.uint8) if a.dtype != torch.float32 else a, b.view(torch.uint8) if b.dtype != torch.float32 else b), name
+    assert float(km.float().abs().mean()) > 0.5
