@@ -28,6 +28,7 @@
 // scale indexing :100-133, mask indexing :222/:268, out-of-range columns attn_utils.cuh:355-381,
 // softmax recurrence attn_utils.cuh:383-488, normalisation :786-840, lse = log2(d) + m (:711-723).
 #include "attn_common.hpp"
+#include <atomic>
 #include <mutex>
 #include <stdlib.h>
 
@@ -641,6 +642,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, G = gridDim.x >> 3;
   const int first = xcd * per, last = min(first + per, p.total);
   unsigned arrivals = 0;
+  bool waiting = true;   // a workgroup that has once waited in vain goes on without waiting for the rest of the launch
   for (int base = first; base < last; base += G) {
     const int vid = base + slot;
     if (vid < last) attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>(p, vid);
@@ -651,9 +653,15 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
       arrivals += (unsigned)G;
       unsigned* c = counters + xcd * PACE_PAD;
       __hip_atomic_fetch_add(c, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      for (int spin = 0; spin < spin_limit; spin++) {
-        if (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= arrivals) break;
-        __builtin_amdgcn_s_sleep(32);
+      if (waiting) {
+        int spin = 0;
+        for (; spin < spin_limit; spin++) {
+          if (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= arrivals) break;
+          __builtin_amdgcn_s_sleep(32);
+        }
+        // its generation is not co-resident (another kernel holds compute units, or the counters are not this
+        // launch's alone): waiting again at every generation would cost the spin limit each time
+        if (spin >= spin_limit && spin_limit > 0) waiting = false;
       }
     }
     __syncthreads();
@@ -662,8 +670,13 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
 
 __global__ void attn_pace_reset_kernel(unsigned* counters) { counters[threadIdx.x] = 0u; }
 
-// counters of the paced kernel: library-owned, one set per GPU (looked up once per device)
-static __device__ __align__(256) unsigned g_pace_counters[8 * PACE_PAD];
+// Counters of the paced kernel: library-owned (looked up once per device), PACE_SETS sets of one counter per XCD.
+// Consecutive paced launches of the process take the sets in turn, so that launches which overlap on one GPU
+// (two streams, two threads) do not zero or count on each other's counters unless more than PACE_SETS of them are
+// in flight at once; even then only the pacing suffers (a workgroup stops waiting after its first timeout).
+constexpr int PACE_SETS = 8;
+static __device__ __align__(256) unsigned g_pace_counters[PACE_SETS * 8 * PACE_PAD];
+static std::atomic<unsigned> g_pace_launches{0};
 constexpr int PACE_MAX_DEVICES = 64;
 struct PaceDevice { unsigned* counters; int cus; };
 static PaceDevice g_pace_dev[PACE_MAX_DEVICES];
@@ -689,7 +702,7 @@ static int pace_device(PaceDevice* out) {
 // The caller's flags decide (PARO_ATTN_PACED / PARO_ATTN_UNPACED); without either, the environment
 // variable PARO_ATTN_PACING (0: never, 1: always) does, and without that the launch is paced when one
 // head's K8 + V8 exceed the 4 MB L2 of an XCD.  PARO_ATTN_PACE_SPINS: rounds (about 1 us each) a workgroup
-// waits for its generation at most (default 4096).
+// waits for its generation at most (default: half the number of key blocks, between 64 and 4096).
 static bool want_pacing(const AttnParams& p, int D) {
   if (p.pacing != 0) return p.pacing > 0;
   if (const char* e = getenv("PARO_ATTN_PACING")) return e[0] == '1';
@@ -710,10 +723,13 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
     const int G = per_cu * (pd.cus / 8);        // workgroups resident on one XCD
     const int per = (p.total + 7) / 8;          // q-blocks per XCD, a contiguous range of (batch, head, q-block)
     if (G > 0 && per > G) {                     // more than one generation: otherwise the plain launch is the same
-      int spins = 4096;
+      // rounds of about 1 us: a q-block of a dense mask takes about 1.3 us per key block, and there is no point in
+      // waiting longer for a generation than half of that
+      int spins = max(64, min(4096, p.nbk / 2));
       if (const char* e = getenv("PARO_ATTN_PACE_SPINS")) spins = atoi(e);
-      hipLaunchKernelGGL(attn_pace_reset_kernel, dim3(1), dim3(8 * PACE_PAD), 0, st, pd.counters);
-      hipLaunchKernelGGL(kern, dim3(8 * G), dim3(128), smem, st, p, pd.counters, per, spins);
+      unsigned* counters = pd.counters + (g_pace_launches.fetch_add(1u) % PACE_SETS) * (8 * PACE_PAD);
+      hipLaunchKernelGGL(attn_pace_reset_kernel, dim3(1), dim3(8 * PACE_PAD), 0, st, counters);
+      hipLaunchKernelGGL(kern, dim3(8 * G), dim3(128), smem, st, p, counters, per, spins);
       PARO_HIP(hipGetLastError());
       return PARO_OK;
     }

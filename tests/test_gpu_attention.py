@@ -337,3 +337,51 @@ def test_paced_launch_is_bit_identical(dev, D, H, N, monkeypatch):
     qattn.attn_sparse_prepacked(q8, k8, v8, vsc, vm, a, qs, ks, D ** -0.5, mask, pacing=False)
     qattn.attn_sparse_prepacked(q8, k8, v8, vsc, vm, b, qs, ks, D ** -0.5, mask, pacing=True)
     assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_paced_launches_that_overlap_on_two_streams(dev):
+    """Two paced launches in flight at once on one GPU (two streams, as a caller that runs the two halves of a
+    classifier-free-guidance batch side by side would have them): each takes its own set of the library's pacing
+    counters, so neither zeroes the other's; the resident workgroups of the second cannot all be co-resident with
+    the first, so its generations stop waiting after one bounded wait.  Results bit-identical to the launches run
+    one after the other, and the pair takes no longer than 1.2 x the two alone plus one wait limit."""
+    import time
+    from paroatten_amd import _qattn_sm80 as qattn
+    from paroatten_amd import quant as Q
+    B, H, N, D = 1, 8, 16384, 128
+    nb = N // 64
+    cases = []
+    for seed in (11, 12):
+        q, k, v = synth.make_qkv_device(B, H, N, D, torch.bfloat16, seed=seed, device=dev)
+        mask = synth.make_block_mask(H, nb, 0.25, seed=seed + 20, device=dev)
+        q8, qs, k8, ks = Q.per_warp_int8(q, k, None, BLKQ=64, WARPQ=32, BLKK=64)
+        v8, vsc, vm = Q.per_channel_fp8(v)
+        cases.append((q8, k8, v8, vsc, vm, qs, ks, mask, torch.empty_like(q), torch.empty_like(q)))
+
+    def launch(c, out):
+        qattn.attn_sparse_prepacked(c[0], c[1], c[2], c[3], c[4], out, c[5], c[6], D ** -0.5, c[7], pacing=True)
+
+    for c in cases:          # one after the other, on the current stream
+        launch(c, c[8])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        for c in cases:
+            launch(c, c[8])
+    torch.cuda.synchronize()
+    serial = (time.perf_counter() - t0) / 5
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(6):     # (the first repetition warms the streams up and is not timed)
+        if rep == 1:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        for c, s in zip(cases, streams):
+            with torch.cuda.stream(s):
+                launch(c, c[9])
+    torch.cuda.synchronize()
+    overlapped = (time.perf_counter() - t0) / 5
+    for c in cases:
+        assert torch.equal(c[8].view(torch.int16), c[9].view(torch.int16))
+        assert torch.isfinite(c[9].float()).all()
+    wait_limit = 128 * 2e-6      # nb / 2 rounds of one to two microseconds
+    assert overlapped <= 1.2 * serial + wait_limit, (overlapped, serial)
