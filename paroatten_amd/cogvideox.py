@@ -15,6 +15,8 @@ return value and `get_time_stats()`.  What changes underneath:
 """
 from __future__ import annotations
 
+import weakref
+
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -54,6 +56,39 @@ class _PathTimer:
         self._pending = keep
 
 
+class _SharedTables:
+    """fp32 (cos, sin) tables in the form the kernels read, derived once per source and shared by every processor
+    of the process: the 40-odd layers of a step all receive the same rotary tensors (Wan rebuilds its `rotary_emb`
+    on every forward, so a cache per processor would convert it 40 times a step and keep 40 copies, ~77 MB each
+    at 720p).  A source is recognised by the identity of its tensor objects (held weakly: an address alone can
+    come back with other contents) and their version counters; the two most recent sources are kept."""
+
+    KEEP = 2
+
+    def __init__(self):
+        self._entries = []   # [(device string, [(weakref, version), ...], cos, sin)], most recent last
+
+    def get(self, src, device, make):
+        dev = str(device)
+        for i, (d, refs, cos, sin) in enumerate(self._entries):
+            if d == dev and len(refs) == len(src) and all(r() is t and t._version == v for t, (r, v) in zip(src, refs)):
+                if i != len(self._entries) - 1:
+                    self._entries.append(self._entries.pop(i))
+                return cos, sin
+        cos, sin = make()
+        cos = cos.to(device=device, dtype=torch.float32).contiguous()
+        sin = sin.to(device=device, dtype=torch.float32).contiguous()
+        self._entries.append((dev, [(weakref.ref(t), t._version) for t in src], cos, sin))
+        del self._entries[:-self.KEEP]
+        return cos, sin
+
+    def clear(self):
+        self._entries = []
+
+
+SHARED_TABLES = _SharedTables()
+
+
 class _ParoProcessorBase:
     """State and helpers shared by the CogVideoX and Wan processors."""
 
@@ -67,8 +102,6 @@ class _ParoProcessorBase:
         self.time_accum = {"total": 0.0}
         self.call_count = 0
         self._orders_cache = {}
-        self._table_cache = (None, None, None)
-        self._table_src = None
         self.i_timestep = 0
         self.i_block = 0
 
@@ -111,18 +144,6 @@ class _ParoProcessorBase:
         if g is None or g[0] * g[1] * g[2] != n_img:
             raise ValueError(f"{n_img} image tokens do not match grid {g}: set the processor's `grid` to (F, H, W)")
         return g
-
-    def _same_source(self, src) -> bool:
-        """True if `src` (a tensor or a tuple of tensors) is what the cached tables were made from: the
-        very same tensor objects, unmodified since.  An address alone would not do: a rotary table that
-        the model rebuilds on every forward can come back at a recycled address with other contents."""
-        old = self._table_src
-        if old is None or len(old) != len(src):
-            return False
-        return all(t is o and t._version == v for t, (o, v) in zip(src, old))
-
-    def _remember_source(self, src):
-        self._table_src = [(t, t._version) for t in src]
 
     @staticmethod
     def _rope_permute(query, key, value, orders, grid, n_text, cos, sin, rotate_key=True):
@@ -169,11 +190,7 @@ class PARO_CogVideoXAttnProcessor2_0(_ParoProcessorBase):
 
     def _tables(self, image_rotary_emb, device):
         cos, sin = image_rotary_emb
-        if self._table_cache[0] != str(device) or not self._same_source((cos, sin)):
-            self._table_cache = (str(device), cos.to(device=device, dtype=torch.float32).contiguous(),
-                                 sin.to(device=device, dtype=torch.float32).contiguous())
-            self._remember_source((cos, sin))
-        return self._table_cache[1], self._table_cache[2]
+        return SHARED_TABLES.get((cos, sin), device, lambda: (cos, sin))
 
     def __call__(self, attn, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,
                  attention_mask: Optional[torch.Tensor] = None,

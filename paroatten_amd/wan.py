@@ -24,7 +24,7 @@ import torch.nn.functional as F
 
 from . import permute as PM
 from . import rope
-from .cogvideox import _ParoProcessorBase
+from .cogvideox import SHARED_TABLES, _ParoProcessorBase
 from .permute import PERMUTATIONS, PERMUTATIONS_INV  # noqa: F401
 
 WAN_GRIDS = {21 * 45 * 80: (21, 45, 80), 21 * 30 * 52: (21, 30, 52)}
@@ -43,13 +43,9 @@ def permute_attn_out(attn_out, permute_plan, i_block, grid=(21, 45, 80), n_text=
 
 class PARO_WanAttnProcessor2_0(_ParoProcessorBase):
     def _tables(self, rotary_emb, device, head_dim):
-        if self._table_cache[0] != str(device) or not self._same_source((rotary_emb,)):
-            freqs = rotary_emb.reshape(-1, head_dim // 2)
-            cos, sin = rope.complex_to_real_tables(freqs)
-            self._table_cache = (str(device), cos.to(device=device, dtype=torch.float32).contiguous(),
-                                 sin.to(device=device, dtype=torch.float32).contiguous())
-            self._remember_source((rotary_emb,))
-        return self._table_cache[1], self._table_cache[2]
+        # (shared by all the processors of the model: the rotary tensor of a step is converted once)
+        return SHARED_TABLES.get((rotary_emb,), device,
+                                 lambda: rope.complex_to_real_tables(rotary_emb.reshape(-1, head_dim // 2)))
 
     def __call__(self, attn, hidden_states: torch.Tensor, encoder_hidden_states: Optional[torch.Tensor] = None,
                  attention_mask: Optional[torch.Tensor] = None, rotary_emb: Optional[torch.Tensor] = None):

@@ -108,3 +108,16 @@ def test_processor_grid_and_table_cache_rules():
     assert a2[0] is not a1[0] and torch.equal(a2[0], cos.float())
     cos2 = cos.clone()                                                     # another object: rebuilt
     assert c._tables((cos2, sin), "cpu")[0] is not a2[0]
+    # the processors of a model share ONE conversion per source (Wan hands every layer the same rotary tensor)
+    from paroatten_amd.cogvideox import SHARED_TABLES
+    c2 = PARO_CogVideoXAttnProcessor2_0()
+    assert c2._tables((cos2, sin), "cpu")[0] is c._tables((cos2, sin), "cpu")[0]
+    freqs = torch.polar(torch.ones(1, 1, 6, 4, dtype=torch.float64), torch.rand(1, 1, 6, 4, dtype=torch.float64))
+    w1, w2 = PARO_WanAttnProcessor2_0(), PARO_WanAttnProcessor2_0()
+    t1 = w1._tables(freqs, "cpu", 8)
+    assert w2._tables(freqs, "cpu", 8)[0] is t1[0] and t1[0].shape == (6, 8)
+    assert len(SHARED_TABLES._entries) <= SHARED_TABLES.KEEP                # bounded: the two most recent sources
+    del freqs                                                               # the source is held weakly
+    import gc
+    gc.collect()
+    assert any(r() is None for _, refs, _, _ in SHARED_TABLES._entries for r, _ in refs)
