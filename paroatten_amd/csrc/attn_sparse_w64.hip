@@ -37,6 +37,15 @@ struct W64Lds {
 
 template <int N> using IC = std::integral_constant<int, N>;
 
+// The lane number, computed where it is needed.  (The rare paths of the loop and the epilogue derive half a
+// dozen values from it; taken from threadIdx they would all be kept in registers across the loop, which has
+// none to spare.  Opaque to the compiler so that it is not hoisted back.)
+__device__ __forceinline__ int lane_here() {
+  int x;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(x));
+  return x;
+}
+
 template <int OUT_DT, bool CAUSAL, bool EXACT>
 __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int vid) {
   using Lds = W64Lds;
@@ -140,22 +149,19 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
       uniform_ptr(p.k8 + b * p.ks_b + hk * p.ks_h), 0, (int)((int64_t)(p.Nk - 1) * p.ks_n + D), 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr(p.v8 + bhk * p.nbk * (int64_t)Lds::VTILE), 0, p.nbk * Lds::VTILE, 0x00020000);
-  int k_goff[4];
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int pos = i * 1024 + lane * 16;  // byte position inside the LDS tile
-    const int row = pos / D, cpos = (pos % D) / 16;
-    // (less the immediate offset i * 1024 that the instruction adds on both sides; row * ks_n >= i * 1024)
-    k_goff[i] = row * (int)p.ks_n + ((cpos ^ Lds::swz(row)) * 16) - i * 1024;
-  }
+  // LDS byte position i * 1024 + lane * 16 of a K tile is row 16 * i + lane / 4, chunk position lane % 4, which
+  // holds chunk (lane % 4) ^ swz(row); swz(row) = (lane / 16) % 4 whatever i is, so the four pieces of a tile share
+  // one per-lane offset and differ by 16 rows less the immediate 1024 that the instruction adds on both sides
+  const int k_goff = (lane >> 2) * (int)p.ks_n + (((lane & 3) ^ Lds::swz(lane >> 2)) * 16);
+  const int k_piece_stride = 16 * (int)p.ks_n - 1024;
   const int v_goff = lane * 16;
   const int k_blk_stride = 64 * (int)p.ks_n;
   auto load_k = [&](int kb, int ST) {  // rows >= Nk read as 0
     uint8_t* base = smem + ST * Lds::KTILE;
-    buffer_load16_lds<0>(k_rsrc, base, k_goff[0], kb * k_blk_stride);
-    buffer_load16_lds<1024>(k_rsrc, base, k_goff[1], kb * k_blk_stride);
-    buffer_load16_lds<2048>(k_rsrc, base, k_goff[2], kb * k_blk_stride);
-    buffer_load16_lds<3072>(k_rsrc, base, k_goff[3], kb * k_blk_stride);
+    buffer_load16_lds<0>(k_rsrc, base, k_goff, kb * k_blk_stride);
+    buffer_load16_lds<1024>(k_rsrc, base, k_goff, kb * k_blk_stride + k_piece_stride);
+    buffer_load16_lds<2048>(k_rsrc, base, k_goff, kb * k_blk_stride + 2 * k_piece_stride);
+    buffer_load16_lds<3072>(k_rsrc, base, k_goff, kb * k_blk_stride + 3 * k_piece_stride);
   };
   auto load_v = [&](int kb, int ST) {
     uint8_t* base = smem + Lds::V_OFF + ST * Lds::VTILE;
@@ -168,7 +174,7 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
   // that issues them in one batch sits behind the CU's address unit, 16 cycles per instruction, for their duration)
   auto load_k_piece = [&](int kb, int ST, auto ic) {
     constexpr int I = decltype(ic)::value;
-    buffer_load16_lds<I * 1024>(k_rsrc, smem + ST * Lds::KTILE, k_goff[I], kb * k_blk_stride);
+    buffer_load16_lds<I * 1024>(k_rsrc, smem + ST * Lds::KTILE, k_goff, kb * k_blk_stride + I * k_piece_stride);
   };
   auto load_v_piece = [&](int kb, int ST, auto ic) {
     constexpr int I = decltype(ic)::value;
@@ -179,18 +185,15 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
   // ---- fragments ------------------------------------------------------------------------------------
   v4i kfrag[4];       // (ks, mt) at ks*2 + mt: row 32*mt + l32, chunk 2*ks + lh at its swizzled position
   v4i vfrag[2][2];    // (dt, mt)
-  int kr_off[4];
-#pragma unroll
-  for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-    for (int mt = 0; mt < 2; mt++) {
-      const int row = 32 * mt + l32;
-      kr_off[ks * 2 + mt] = row * D + (((2 * ks + lh) ^ Lds::swz(row)) * 16);
-    }
+  // row 32*mt + l32 has the swizzle of row l32; chunk 2*ks + lh sits at position (2*ks + lh) ^ swz: the two k-steps
+  // differ in bit 1 of the position (32 bytes), the two row tiles by 2048 bytes (an immediate offset)
+  const int kr_0 = l32 * D + ((lh ^ Lds::swz(l32)) * 16);
+  const int kr_1 = kr_0 ^ 32;
   const int vr_base = Lds::V_OFF + lane * 16;
   auto read_k_frags = [&](int ST) {
 #pragma unroll
-    for (int i = 0; i < 4; i++) kfrag[i] = *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + kr_off[i]);
+    for (int i = 0; i < 4; i++)
+      kfrag[i] = *reinterpret_cast<const v4i*>(smem + ST * Lds::KTILE + ((i >> 1) ? kr_1 : kr_0) + (i & 1) * 2048);
   };
   auto read_v_frags = [&](int ST) {
 #pragma unroll
@@ -252,8 +255,9 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
     if (edge) {
       int kb_e = kb;
       asm volatile("" : "+s"(kb_e));   // opaque: otherwise 32 lane masks are hoisted into scalar registers
-      int thr = p.Nk - kb_e * 64 - 4 * lh;
-      if constexpr (CAUSAL) thr = min(thr, qrow[hf] + 1 - kb_e * 64 - 4 * lh);
+      const int ln = lane_here();
+      int thr = p.Nk - kb_e * 64 - 4 * (ln >> 5);
+      if constexpr (CAUSAL) thr = min(thr, qb * 64 + hf * 32 + (ln & 31) + 1 - kb_e * 64 - 4 * (ln >> 5));
 #pragma unroll
       for (int mt = 0; mt < 2; mt++)
 #pragma unroll
@@ -292,7 +296,7 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
     m_off[hf] = P_EXP_OFFSET - m_new;
     m_off8[hf] = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT + 0.5f) * FAST_FIELD_SCALE;
     d_acc[hf][0] *= alpha;                                    // lanes 0..15: q-row lane
-    d_acc[hf][1] *= __shfl(alpha, (lane & 15) + 16, 64);      // and q-row lane + 16
+    d_acc[hf][1] *= __shfl(alpha, (lane_here() & 15) + 16, 64);   // and q-row lane + 16
 #pragma unroll
     for (int dt = 0; dt < 2; dt++)
 #pragma unroll
@@ -353,12 +357,16 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
   int kb_1 = __builtin_amdgcn_readfirstlane((int)klist[1]);
   int kb_2 = __builtin_amdgcn_readfirstlane((int)klist[2]);
   int kb_3 = __builtin_amdgcn_readfirstlane((int)klist[3]);
+  // (the q scales are the same in every lane: scalar registers from here on)
+  qsc[0] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(qsc[0])));
+  qsc[1] = __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(qsc[1])));
 
   // One phase.  X: the half whose products are issued (S_X of the next block, O_X of this one); Y = 1 - X: the
   // half whose weights are computed, from the scores of block list entry `yi` (block number kb_y).  xi: list
-  // entry of the block whose weights pf[X] are waiting to be accepted.  LAST: no next block.
+  // entry of the block whose weights pf[X] are waiting to be accepted.  LAST: no next block.  (The first block's
+  // maxima are taken in the prologue: no phase has to ask whether it is the first.)
   // after_qk / after_pv: hooks that read the next fragments once the products using the old ones are issued.
-  auto phase = [&](auto xc, auto lastc, int xi, int yi, int kb_y, bool first_y, auto&& after_qk, auto&& after_pv,
+  auto phase = [&](auto xc, auto lastc, int xi, int yi, int kb_y, auto&& after_qk, auto&& after_pv,
                    auto&& piece) {
     constexpr int X = decltype(xc)::value, Y = 1 - X;
     constexpr bool LAST = decltype(lastc)::value != 0;
@@ -372,8 +380,6 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
       if constexpr (EXACT) {
         const float m_blk = block_max(yc, c);
         if (__ballot(m_blk > m_thr[Y]) != 0ull) apply_refresh(yc, m_blk);
-      } else {
-        if (first_y) apply_refresh(yc, block_max(yc, c));
       }
       affine(yc, c, cs, bs);
       word_fma(yc, ub, 0, cs, bs);
@@ -468,10 +474,14 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
   read_k_frags(1);
   read_v_frags(0);
   {
-    const float c0 = qsc[0] * clist[0];
+    // the first block gives both halves their first maximum (the fast path does not search one again unless a
+    // weight overflows); half A's weights of it are due before the loop
+    const float ks0 = clist[0];
     mask_edge(IC<0>{}, kb_c);
-    apply_refresh(IC<0>{}, block_max(IC<0>{}, c0));
-    all_words(IC<0>{}, c0);
+    mask_edge(IC<1>{}, kb_c);
+    apply_refresh(IC<0>{}, block_max(IC<0>{}, qsc[0] * ks0));
+    if constexpr (!EXACT) apply_refresh(IC<1>{}, block_max(IC<1>{}, qsc[1] * ks0));
+    all_words(IC<0>{}, qsc[0] * ks0);
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 
@@ -480,9 +490,9 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
     constexpr int ST = decltype(stc)::value;
     const int kidx_v = (int)klist[it + 4];
     __builtin_amdgcn_sched_barrier(0);
-    phase(IC<0>{}, IC<0>{}, it, it, kb_c, it == 0, nothing, nothing,
+    phase(IC<0>{}, IC<0>{}, it, it, kb_c, nothing, nothing,
           [&](auto ic) { load_k_piece(kb_3, ST ^ 1, ic); });   // K(it+3) into the stage K(it+1) has left
-    phase(IC<1>{}, IC<0>{}, it, it + 1, kb_1, false,
+    phase(IC<1>{}, IC<0>{}, it, it + 1, kb_1,
           [&]() {   // K(it+2) and V(it+1) have landed: everything older than the last eight requests has
             asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS_PER_IT) : "memory");
             read_k_frags(ST);
@@ -501,22 +511,24 @@ __device__ __forceinline__ void attn_qblock_w64(const AttnParams& p, const int v
     body(IC<1>{}, it + 1);
   }
   // the last kept block: O += V.P of both halves and the weights of half B
-  phase(IC<0>{}, IC<1>{}, last, last, kb_c, last == 0, nothing, nothing, no_piece);
-  phase(IC<1>{}, IC<1>{}, last, last, kb_c, false, nothing, nothing, no_piece);
+  phase(IC<0>{}, IC<1>{}, last, last, kb_c, nothing, nothing, no_piece);
+  phase(IC<1>{}, IC<1>{}, last, last, kb_c, nothing, nothing, no_piece);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // DMA of the padded tail blocks: nobody reads it
 
   // ---- epilogue: O = O~/d * v_scale + v_mean ------------------------------------------------------------
+  const int ln = lane_here(), e32 = ln & 31, eh = ln >> 5;
 #pragma unroll
   for (int hf = 0; hf < 2; hf++) {
-    const float d_lo = __shfl(d_acc[hf][0], l32 & 15, 64), d_hi = __shfl(d_acc[hf][1], l32 & 15, 64);
-    const float inv = 1.0f / (l32 < 16 ? d_lo : d_hi);
-    if (qrow[hf] < p.Nq) {
-      unsigned short* outp = out_row_ptr(qrow[hf]);
+    const float d_lo = __shfl(d_acc[hf][0], e32 & 15, 64), d_hi = __shfl(d_acc[hf][1], e32 & 15, 64);
+    const float inv = 1.0f / (e32 < 16 ? d_lo : d_hi);
+    const int row = qb * 64 + hf * 32 + e32;
+    if (row < p.Nq) {
+      unsigned short* outp = out_row_ptr(row);
 #pragma unroll
       for (int dt = 0; dt < 2; dt++) {
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-          const int ch = 32 * dt + 8 * g + 4 * lh;
+          const int ch = 32 * dt + 8 * g + 4 * eh;
           const v4f sc = *reinterpret_cast<const v4f*>(epi + ch);
           const v4f mn = *reinterpret_cast<const v4f*>(epi + D + ch);
           unsigned short r[4];
