@@ -454,6 +454,11 @@ def main():
         timed("prepare_fused_rope_permute_quant_fp8",
               lambda: PM.rope_permute_quant(q, k, v, orders, wl.grid, wl.n_text, cos, sin, km=km), el * (2 + 2 + 4) + el * 3)
         timed("rope_k_mean", lambda: PM.rope_k_mean(k, wl.grid, wl.n_text, cos, sin), el * 2)
+        # what the processors call when K smoothing is on: the rotated K mean inside the preparation (K read
+        # twice, V twice, Q once)
+        timed("prepare_with_k_mean",
+              lambda: PM.rope_permute_quant(q, k, v, orders, wl.grid, wl.n_text, cos, sin, km="mean"),
+              el * (2 + 4 + 4) + el * 3)
         timed("permute_inverse_o", lambda: PM.permute_inverse(out, orders, wl.grid, wl.n_text), 2 * el * 2)
         # the same work as separate kernels (what the fused pass replaces)
         timed("rope_permute_qkv", lambda: PM.rope_permute(q, k, v, orders, wl.grid, wl.n_text, cos, sin), 3 * 2 * el * 2)
@@ -474,8 +479,7 @@ def main():
         unperm = (orders, wl.grid, wl.n_text)
 
         def whole_path():
-            kmean = PM.rope_k_mean(k, wl.grid, wl.n_text, cos, sin)
-            ops = PM.rope_permute_quant(q, k, v, orders, wl.grid, wl.n_text, cos, sin, km=kmean)
+            ops = PM.rope_permute_quant(q, k, v, orders, wl.grid, wl.n_text, cos, sin, km="mean")
             qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, token_major.transpose(1, 2),
                                         ops.q_scale, ops.k_scale, sm_scale, head_mask, unpermute=unperm)
 

@@ -635,10 +635,21 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
 // neighbours in the key sequence.  The meeting point between generations only paces: a workgroup that
 // has waited `spin_limit` rounds goes on regardless, so the kernel finishes whatever the residency or
 // the state of the counters (they are zeroed by a small launch in front of this one).
+//
+// A workgroup goes on when all but `slack` of the XCD's workgroups have arrived: the last arrivals of a
+// generation do not hold the others up, and since those never wait themselves they do not fall further behind.
+// What matters for the L2 is that the workgroups stay within the part of the head that it holds, not that they
+// start in the same microsecond; and a generation that starts all at once also runs all its prologues and
+// epilogues at once, with nothing else on the compute unit to cover them.  (Measured on a mask whose rows hold
+// 154 +- 10 and 236 +- 14 kept blocks: waiting for all, 38.8 % / 40.6 % of the matrix peak at Wan 480p / 720p;
+// for all but a quarter 40.8 % / 41.7 %; for all but a half 41.2 % / 40.3 %.  Building the generations from
+// q-blocks of equal length, sorted by a pre-pass over the mask, changed nothing: a workgroup that waits leaves
+// the matrix pipe to its neighbours on the compute unit, so the waiting itself costs little.)
 constexpr int PACE_PAD = 32;   // counters 128 bytes apart: one per XCD
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
 __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
-    attn_sparse_paced_kernel(const AttnParams p, unsigned* __restrict__ counters, const int per, const int spin_limit) {
+    attn_sparse_paced_kernel(const AttnParams p, unsigned* __restrict__ counters, const int per, const int spin_limit,
+                             const int slack) {
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, G = gridDim.x >> 3;
   const int first = xcd * per, last = min(first + per, p.total);
   unsigned arrivals = 0;
@@ -656,7 +667,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
       if (waiting) {
         int spin = 0;
         for (; spin < spin_limit; spin++) {
-          if (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= arrivals) break;
+          if (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + (unsigned)slack >= arrivals) break;
           __builtin_amdgcn_s_sleep(32);
         }
         // its generation is not co-resident (another kernel holds compute units, or the counters are not this
@@ -703,6 +714,8 @@ static int pace_device(PaceDevice* out) {
 // variable PARO_ATTN_PACING (0: never, 1: always) does, and without that the launch is paced when one
 // head's K8 + V8 exceed the 4 MB L2 of an XCD.  PARO_ATTN_PACE_SPINS: rounds (about 1 us each) a workgroup
 // waits for its generation at most (default: half the number of key blocks, between 64 and 4096).
+// PARO_ATTN_PACE_SLACK: how many of an XCD's resident workgroups a generation does not wait for (default: the
+// share of the head's K8 + V8 that the L2 holds, at most half of them).
 static bool want_pacing(const AttnParams& p, int D) {
   if (p.pacing != 0) return p.pacing > 0;
   if (const char* e = getenv("PARO_ATTN_PACING")) return e[0] == '1';
@@ -727,9 +740,13 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
       // waiting longer for a generation than half of that
       int spins = max(64, min(4096, p.nbk / 2));
       if (const char* e = getenv("PARO_ATTN_PACE_SPINS")) spins = atoi(e);
+      // stragglers within the L2's share of the head still find their tiles: that many need not be waited for
+      const int64_t head_bytes = (int64_t)p.nbk * 64 * D * 2;
+      int slack = (int)min((int64_t)G / 2, (int64_t)G * ((int64_t)4 << 20) / head_bytes);
+      if (const char* e = getenv("PARO_ATTN_PACE_SLACK")) slack = max(0, min(G - 1, atoi(e)));
       unsigned* counters = pd.counters + (g_pace_launches.fetch_add(1u) % PACE_SETS) * (8 * PACE_PAD);
       hipLaunchKernelGGL(attn_pace_reset_kernel, dim3(1), dim3(8 * PACE_PAD), 0, st, counters);
-      hipLaunchKernelGGL(kern, dim3(8 * G), dim3(128), smem, st, p, counters, per, spins);
+      hipLaunchKernelGGL(kern, dim3(8 * G), dim3(128), smem, st, p, counters, per, spins, slack);
       PARO_HIP(hipGetLastError());
       return PARO_OK;
     }
