@@ -51,9 +51,9 @@ WORKLOAD_DENSITIES = {
 # CogVideoX: the same at every density (one head's K8 + V8 stay in the L2).  Wan: L2 fills, with the paced
 # launch; they vary by tens of percent from box to box at 720p, where a head is five times the L2.
 ATTN_TRAFFIC_BYTES = {
-    "cogvideox5b": int((167468 * 2.0 + 213796 * 1.0) * 1024),
-    "wan14b_480p": int((744582 * 2.0 + 328686 * 1.0) * 1024),
-    "wan14b_720p": int((12405556 * 2.0 + 771465 * 1.0) * 1024),
+    "cogvideox5b": int((169381 * 2.0 + 213315 * 1.0) * 1024),
+    "wan14b_480p": int((1218830 * 2.0 + 335512 * 1.0) * 1024),
+    "wan14b_720p": int((16747800 * 2.0 + 813568 * 1.0) * 1024),
 }
 
 
@@ -435,7 +435,8 @@ def main():
         "peak": PEAK_MFMA_TOPS,
         "unit": "TOP/s",
         "frac": round(achieved / PEAK_MFMA_TOPS, 4),
-        "traffic": ATTN_TRAFFIC_BYTES.get(args.workload) if args.pacing == "auto" and not args.zero_operands else None,
+        "traffic": (ATTN_TRAFFIC_BYTES.get(args.workload)
+                    if args.pacing == "auto" and not args.zero_operands and not args.two_waves else None),
         "ops_per_launch": hk["kept_blocks"] * 4.0 * 64 * 64 * D,
         "avg_launch_ms": hk["attn_kernel_ms"],
     }

@@ -641,8 +641,9 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
 // What matters for the L2 is that the workgroups stay within the part of the head that it holds, not that they
 // start in the same microsecond; and a generation that starts all at once also runs all its prologues and
 // epilogues at once, with nothing else on the compute unit to cover them.  (Measured on a mask whose rows hold
-// 154 +- 10 and 236 +- 14 kept blocks: waiting for all, 38.8 % / 40.6 % of the matrix peak at Wan 480p / 720p;
-// for all but a quarter 40.8 % / 41.7 %; for all but a half 41.2 % / 40.3 %.  Building the generations from
+// 154 +- 10 and 236 +- 14 kept blocks: waiting for all, 38.3 % / 38.9 % of the matrix peak at Wan 480p / 720p;
+// for all but an eighth 39.6 % / 39.6 %; for all but a quarter 40.0 % / 39.2 %; for all but a half 39.6 % /
+// 37.2 %, the L2 fills growing from 1.6 to 8.7 GB and from 29 to 75 GB per launch.  Building the generations from
 // q-blocks of equal length, sorted by a pre-pass over the mask, changed nothing: a workgroup that waits leaves
 // the matrix pipe to its neighbours on the compute unit, so the waiting itself costs little.)
 constexpr int PACE_PAD = 32;   // counters 128 bytes apart: one per XCD
@@ -714,8 +715,8 @@ static int pace_device(PaceDevice* out) {
 // variable PARO_ATTN_PACING (0: never, 1: always) does, and without that the launch is paced when one
 // head's K8 + V8 exceed the 4 MB L2 of an XCD.  PARO_ATTN_PACE_SPINS: rounds (about 1 us each) a workgroup
 // waits for its generation at most (default: half the number of key blocks, between 64 and 4096).
-// PARO_ATTN_PACE_SLACK: how many of an XCD's resident workgroups a generation does not wait for (default: the
-// share of the head's K8 + V8 that the L2 holds, at most half of them).
+// PARO_ATTN_PACE_SLACK: how many of an XCD's resident workgroups a generation does not wait for (default: half
+// the share of the head's K8 + V8 that the L2 holds, at most a quarter of them).
 static bool want_pacing(const AttnParams& p, int D) {
   if (p.pacing != 0) return p.pacing > 0;
   if (const char* e = getenv("PARO_ATTN_PACING")) return e[0] == '1';
@@ -740,9 +741,11 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
       // waiting longer for a generation than half of that
       int spins = max(64, min(4096, p.nbk / 2));
       if (const char* e = getenv("PARO_ATTN_PACE_SPINS")) spins = atoi(e);
-      // stragglers within the L2's share of the head still find their tiles: that many need not be waited for
+      // stragglers within half of the L2's share of the head still find their tiles: that many need not be waited
+      // for (measured optimum on two boxes: about 32 of 128 at Wan 480p, 8.4 MB per head, and 8 to 16 at 720p,
+      // 19.4 MB; beyond that the L2 fills grow quickly, 1.6 -> 8.7 GB per launch at 480p from 16 to 64)
       const int64_t head_bytes = (int64_t)p.nbk * 64 * D * 2;
-      int slack = (int)min((int64_t)G / 2, (int64_t)G * ((int64_t)4 << 20) / head_bytes);
+      int slack = (int)min((int64_t)G / 4, (int64_t)G * ((int64_t)2 << 20) / head_bytes);
       if (const char* e = getenv("PARO_ATTN_PACE_SLACK")) slack = max(0, min(G - 1, atoi(e)));
       unsigned* counters = pd.counters + (g_pace_launches.fetch_add(1u) % PACE_SETS) * (8 * PACE_PAD);
       hipLaunchKernelGGL(attn_pace_reset_kernel, dim3(1), dim3(8 * PACE_PAD), 0, st, counters);
