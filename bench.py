@@ -413,6 +413,20 @@ def main():
             if D == 64:
                 t_2w = event_time_ms(lambda: attn_only(masks[d], attn_flags | L.PARO_ATTN_TWO_WAVES), reps, 2)
                 dens[str(d)]["attn_kernel_ms_two_waves"] = round(t_2w, 4)
+            if not args.zero_operands:
+                # the accuracy mode (float16 P.V product, what the reference's kernel computes): its own V tiles
+                from paroatten_amd import _qattn_sm80 as QA
+                v16 = QA.v_f16_tiles(vp)
+
+                def attn_pv16():
+                    L.check(lib.paro_attn_sparse_fwd(
+                        L.ptr(aq8), L.ptr(ak8), L.ptr(v16), L.ptr(qs), L.ptr(ks), None, None, L.ptr(masks[d]), 0,
+                        L.ptr(out), L.DTYPE_CODE[out.dtype], None, None, B, H, H, N, N, D,
+                        q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
+                        out.stride(0), out.stride(1), out.stride(2), sm_scale, 0, L.PARO_ATTN_PV_F16, L.stream_of(out)))
+                t_16 = event_time_ms(attn_pv16, max(10, reps // 4), 2)
+                dens[str(d)]["attn_kernel_ms_pv_f16"] = round(t_16, 4)
+                del v16
     if not args.headline_only:
         # the same number of blocks per row as one contiguous run round the diagonal (not a benchmark
         # configuration: it shows what the mask FAMILY costs when a head's K8 + V8 exceed the L2)

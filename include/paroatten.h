@@ -50,6 +50,14 @@ extern "C" {
 #define PARO_ATTN_TWO_WAVES 8 /* kernel form, results are bit-identical either way: two waves per 64-row q-block
                                  (32 q-rows each) also where the library would pick the one-wave-per-q-block
                                  kernel (head size 64, no lse, plain launch), which is the faster of the two there */
+#define PARO_ATTN_PV_F16 16   /* accuracy mode: the P.V product in float16 with fp32 accumulation, as the reference's
+                                 qk_int8_sv_f16_accum_f16_attn computes it (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:263-391),
+                                 instead of FP8 e4m3 P and V.  True exponentials; V as given (no per-channel scale, no
+                                 mean).  For paro_attn_sparse_fwd / _unpermute_fwd the `v8` argument then points at
+                                 paro_v_f16_pack's tiles and v_scale / v_mean may be NULL; paro_qk_int8_sv_f16_attn
+                                 packs them into its workspace itself (paro_attn_workspace_bytes_for).  Plain launch
+                                 only; about half the speed of the default (the matrix pipe runs float16 at half the
+                                 FP8 rate). */
 
 /* Version of this ABI (bumped when a signature changes). */
 int paro_abi_version(void);
@@ -102,6 +110,19 @@ int paro_v_fp8_pack(const void* v, int dtype, uint8_t* v8, float* v_scale, float
                     int B, int Hkv, int N, int D,
                     int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n,
                     int smooth, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * (2a') V -> float16 tiles for the attention's accuracy mode (PARO_ATTN_PV_F16).  Stands in for the
+ * float16 V operand the reference's kernel reads as it is (value.to(float16) in its callers,
+ * paroattention/core.py:150-160): values unchanged (bfloat16 inputs converted to float16, round to nearest
+ * even), no scale, no mean; only the order differs.
+ * v [B,Hkv,N,D] 16-bit.  v16: paro_v_f16_bytes() bytes.  Tile order: halfword
+ * v16[((b*Hkv+h)*nb + kb)*64*D + ((dt*4 + s)*64 + lane)*8 + e] holds token
+ * kb*64 + 32*(s/2) + 16*(s%2) + 8*(e/4) + 4*(lane/32) + e%4, channel 32*dt + lane%32 (tokens >= N are 0).
+ * ------------------------------------------------------------------------------------------- */
+int64_t paro_v_f16_bytes(int B, int Hkv, int N, int D);
+int paro_v_f16_pack(const void* v, int dtype, void* v16, int B, int Hkv, int N, int D,
+                    int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_n, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * (2b) Block-sparse attention: INT8 Q.K^T on i8 MFMA (exact int32), online base-2 softmax,
@@ -167,6 +188,8 @@ int paro_attn_sparse_unpermute_fwd(const int8_t* q8, const int8_t* k8, const uin
  * workspace: paro_attn_workspace_bytes() bytes of device memory (256-byte aligned).
  * ------------------------------------------------------------------------------------------- */
 int64_t paro_attn_workspace_bytes(int B, int Hkv, int Nk, int D);
+/* The same for a call with the given flags (PARO_ATTN_PV_F16 needs float16 tiles of V instead). */
+int64_t paro_attn_workspace_bytes_for(int B, int Hkv, int Nk, int D, int flags);
 int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, const void* v, int v_dtype,
                              void* out, int out_dtype,
                              const float* q_scale, const float* k_scale,

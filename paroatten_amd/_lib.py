@@ -23,6 +23,7 @@ PARO_ATTN_EXACT_EXP = 1
 PARO_ATTN_PACED = 2
 PARO_ATTN_UNPACED = 4
 PARO_ATTN_TWO_WAVES = 8
+PARO_ATTN_PV_F16 = 16
 
 DTYPE_CODE = {torch.float16: 0, torch.bfloat16: 1}
 
@@ -48,6 +49,9 @@ SIGNATURES = {
                                                _L, _L, _L, _L, _L, _L, _L, _L, _L, _F, _I, _I,
                                                _P, _I, _I, _I, _I, _P]),
     "paro_attn_workspace_bytes": (c_int64, [_I, _I, _I, _I]),
+    "paro_attn_workspace_bytes_for": (c_int64, [_I, _I, _I, _I, _I]),
+    "paro_v_f16_bytes": (c_int64, [_I, _I, _I, _I]),
+    "paro_v_f16_pack": (c_int, [_P, _I, _P, _I, _I, _I, _I, _L, _L, _L, _P]),
     "paro_qk_int8_sv_f16_attn": (c_int, [_P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _P, _P, _L,
                                          _I, _I, _I, _I, _I, _I,
                                          _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,

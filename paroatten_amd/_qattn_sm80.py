@@ -11,6 +11,9 @@ Differences, all relaxations or added checks:
   * `value` may be float16 (as in the reference) or bfloat16 (saves the caller's `.to(float16)`);
   * keyword `exact_exp=True` evaluates the softmax exponentials in fp32 before the FP8 rounding instead
     of building the e4m3 byte directly (slower, slightly more accurate; always on with return_lse);
+  * keyword `pv_f16=True` is the accuracy mode (PARO_ATTN_PV_F16): the P.V product in float16 with fp32
+    accumulation, as the reference's kernel of this name computes it, instead of FP8 e4m3 P and V: true
+    exponentials, V as given (smooth_v has nothing to act on); about half the speed;
   * keyword `pacing=True/False` picks the launch form of the attention kernel (see PARO_ATTN_PACED in
     include/paroatten.h; bit-identical results), None leaves it to the library;
   * `sparse` IS validated (the reference reads it through a raw pointer unchecked): bool or uint8,
@@ -31,10 +34,13 @@ def _chk(cond, msg):
         raise RuntimeError(msg)
 
 
-def _flags(exact_exp, pacing, two_waves=False):
+def _flags(exact_exp, pacing, two_waves=False, pv_f16=False):
     """pacing: None (the library chooses), True (PARO_ATTN_PACED) or False (PARO_ATTN_UNPACED); two_waves:
-    PARO_ATTN_TWO_WAVES.  Launch and kernel form only: results are bit-identical."""
+    PARO_ATTN_TWO_WAVES.  Launch and kernel form only: results are bit-identical.  pv_f16: PARO_ATTN_PV_F16, the
+    float16 P.V product."""
     f = _lib.PARO_ATTN_EXACT_EXP if exact_exp else 0
+    if pv_f16:
+        f |= _lib.PARO_ATTN_PV_F16
     if pacing is not None:
         f |= _lib.PARO_ATTN_PACED if pacing else _lib.PARO_ATTN_UNPACED
     if two_waves:
@@ -42,13 +48,29 @@ def _flags(exact_exp, pacing, two_waves=False):
     return f
 
 
-def workspace_bytes(B, Hkv, Nk, D):
+def workspace_bytes(B, Hkv, Nk, D, pv_f16=False):
+    if pv_f16:
+        return int(load().paro_attn_workspace_bytes_for(B, Hkv, Nk, D, _lib.PARO_ATTN_PV_F16))
     return int(load().paro_attn_workspace_bytes(B, Hkv, Nk, D))
+
+
+def v_f16_tiles(value, tensor_layout="HND"):
+    """V [B,Hkv,N,D] ("HND") or [B,N,Hkv,D] ("NHD"), float16 or bfloat16 -> the float16 tiles that the attention
+    kernel's accuracy mode reads (paro_v_f16_pack): uint8 tensor of paro_v_f16_bytes() bytes."""
+    _chk(value.is_cuda and value.dim() == 4 and value.stride(-1) == 1 and value.dtype in _lib.DTYPE_CODE,
+         "Tensor value must be a float16/bfloat16 GPU tensor [B,H,N,D] with a contiguous last dimension")
+    if tensor_layout == "NHD":
+        value = value.transpose(1, 2)
+    B, Hkv, N, D = value.shape
+    out = torch.empty(int(load().paro_v_f16_bytes(B, Hkv, N, D)), dtype=torch.uint8, device=value.device)
+    _lib.on(value).paro_v_f16_pack(ptr(value), _lib.DTYPE_CODE[value.dtype], ptr(out), B, Hkv, N, D,
+                                   value.stride(0), value.stride(1), value.stride(2), stream_of(value))
+    return out
 
 
 def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_scale, tensor_layout, is_causal,
                                   qk_quant_gran, sm_scale, return_lse, sparse, *, smooth_v=True, exact_exp=False,
-                                  workspace=None, pacing=None, two_waves=False):
+                                  workspace=None, pacing=None, two_waves=False, pv_f16=False):
     for t, n in ((query, "query"), (key, "key"), (value, "value"), (output, "output"),
                  (query_scale, "query_scale"), (key_scale, "key_scale")):
         _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
@@ -113,7 +135,7 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
     lse = torch.empty(0)
     if return_lse:
         lse = torch.empty((B, H, Nq), dtype=torch.float32, device=query.device)
-    need = workspace_bytes(B, Hkv, Nk, D)
+    need = workspace_bytes(B, Hkv, Nk, D, pv_f16)
     if workspace is None:
         workspace = torch.empty(need, dtype=torch.uint8, device=query.device)
     else:
@@ -129,19 +151,22 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
         value.stride(0), value.stride(sh), value.stride(sn),
         output.stride(0), output.stride(sh), output.stride(sn),
         tensor_layout, is_causal, qk_quant_gran, float(sm_scale), 1 if smooth_v else 0,
-        _flags(exact_exp, pacing, two_waves), stream_of(query))
+        _flags(exact_exp, pacing, two_waves, pv_f16), stream_of(query))
     return lse
 
 
 def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_scale, sm_scale, sparse,
                           is_causal=0, return_lse=0, exact_exp=False, unpermute=None, pacing=None,
-                          two_waves=False):
+                          two_waves=False, pv_f16=False):
     """The attention kernel alone, on operands that are already in its formats (HND, contiguous):
     q8/k8 int8 [B,H,N,D] / [B,Hkv,Nk,D], v8 = FP8 tiles from paro_v_fp8_pack or the fused
-    preparation, v_scale / v_mean f32 [B,Hkv,D] (v_mean None: V was not mean-smoothed).  No
+    preparation, v_scale / v_mean f32 [B,Hkv,D] (v_mean None: V was not mean-smoothed).  With pv_f16=True
+    v8 holds the float16 tiles of v_f16_tiles() and v_scale / v_mean may be None.  No
     counterpart in the reference, whose extension converts V on every call."""
     for t, n in ((q8, "query"), (k8, "key"), (v8, "value"), (output, "output"), (query_scale, "query_scale"),
                  (key_scale, "key_scale"), (v_scale, "v_scale"), (sparse, "sparse")):
+        if t is None and pv_f16 and n == "v_scale":
+            continue
         _chk(t.is_cuda, f"Tensor {n} must be on CUDA")
         _chk(t.is_contiguous() or n == "output", f"Tensor {n} must be contiguous")
     _chk(q8.dtype == torch.int8 and k8.dtype == torch.int8, "Tensor query/key must have dtype (torch::kInt8)")
@@ -153,10 +178,16 @@ def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_
     if H % Hkv != 0:
         raise ValueError(f"num_qo_heads ({H}) must be divisible by num_kv_heads ({Hkv})")
     nbq, nbk = (Nq + 63) // 64, (Nk + 63) // 64
-    _chk(v8.numel() * v8.element_size() == load().paro_v_fp8_bytes(B, Hkv, Nk, D), "Tensor value has the wrong size for FP8 tiles")
+    if pv_f16:
+        _chk(v8.numel() * v8.element_size() == load().paro_v_f16_bytes(B, Hkv, Nk, D),
+             "Tensor value has the wrong size for float16 tiles")
+    else:
+        _chk(v8.numel() * v8.element_size() == load().paro_v_fp8_bytes(B, Hkv, Nk, D),
+             "Tensor value has the wrong size for FP8 tiles")
     _chk(tuple(query_scale.shape) == (B, H, nbq * 2) and tuple(key_scale.shape) == (B, Hkv, nbk),
          "Tensor query_scale / key_scale must have shapes (B, H, 2*nbq) / (B, Hkv, nbk)")
-    _chk(tuple(v_scale.shape) == (B, Hkv, D) and (v_mean is None or tuple(v_mean.shape) == (B, Hkv, D)),
+    _chk((v_scale is None and pv_f16 or tuple(v_scale.shape) == (B, Hkv, D))
+         and (v_mean is None or tuple(v_mean.shape) == (B, Hkv, D)),
          "Tensor v_scale / v_mean must have shape (B, Hkv, head_dim)")
     _chk(tuple(output.shape) == (B, H, Nq, D) and output.stride(-1) == 1 and output.dtype in _lib.DTYPE_CODE,
          "Tensor output must be float16/bfloat16 [B,H,N,D] with a contiguous last dimension")
@@ -168,7 +199,7 @@ def attn_sparse_prepacked(q8, k8, v8, v_scale, v_mean, output, query_scale, key_
         _chk(tuple(sparse.shape) == (H, nbq, nbk), f"Tensor sparse must have shape ([{B},] {H}, {nbq}, {nbk})")
         sparse_bs = 0
     lse = torch.empty((B, H, Nq), dtype=torch.float32, device=q8.device) if return_lse else torch.empty(0)
-    flags = _flags(exact_exp, pacing, two_waves)
+    flags = _flags(exact_exp, pacing, two_waves, pv_f16)
     strides = (q8.stride(0), q8.stride(1), q8.stride(2), k8.stride(0), k8.stride(1), k8.stride(2),
                output.stride(0), output.stride(1), output.stride(2))
     if unpermute is None:

@@ -22,7 +22,7 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIBDIR = PKG / "lib"
 LIB = LIBDIR / "libparoatten_hip.so"
-SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "v_channel.hip", "rope_permute.hip", "fused_prep.hip", "mask_bits.hip", "attn_sparse.hip", "attn_sparse_w64.hip"]
+SOURCES = ["paro_common.hip", "quant_int8.hip", "v_fp8.hip", "v_channel.hip", "rope_permute.hip", "fused_prep.hip", "mask_bits.hip", "attn_sparse.hip", "attn_sparse_w64.hip", "attn_sparse_pv16.hip"]
 ARCH = "gfx950"
 # measurement aids behind bench.py --mfma-ceiling / --proxy-ceiling: a library of their own (include/paroatten_diag.h),
 # outside the drop-in boundary

@@ -33,7 +33,7 @@ def paroattn(q, k, v, tensor_layout: str = "HND", is_causal: bool = False, sm_sc
 def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", is_causal: bool = False,
                                   qk_quant_gran: str = "per_warp", sm_scale: Optional[float] = None,
                                   return_lse: bool = False, smooth_k: bool = False, smooth_v: bool = True,
-                                  exact_exp: bool = False, two_waves: bool = False, **kwargs: Any):
+                                  exact_exp: bool = False, two_waves: bool = False, pv_f16: bool = False, **kwargs: Any):
     """INT8 Q.K^T, FP8 P.V block-sparse attention.
 
     q [B,Hq,Nq,D] / k, v [B,Hkv,Nk,D] ("HND") or [B,N,H,D] ("NHD"), float16 or bfloat16, same
@@ -43,7 +43,10 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
     smooth_k subtracts the per-(batch,head) token mean of K before quantisation (softmax is
     invariant to it); smooth_v does the same for V inside the FP8 conversion and adds the mean back;
     exact_exp trades speed for fp32-evaluated softmax exponentials (see _qattn_sm80); two_waves picks the
-    two-waves-per-q-block kernel where the library would take the one-wave one (bit-identical results).
+    two-waves-per-q-block kernel where the library would take the one-wave one (bit-identical results);
+    pv_f16 is the accuracy mode: the P.V product in float16 with fp32 accumulation, as the reference computes
+    it (qk_int8_sv_f16_accum_f16_attn), instead of FP8 e4m3: about half the speed, float16 instead of e4m3 error
+    on rows that a few keys dominate.
     """
     dtype = q.dtype
     assert q.is_cuda, "Input tensors must be on cuda."
@@ -83,7 +86,7 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
         lse = qattn.qk_int8_sv_f16_accum_f16_attn(q_int8, k_int8, v, o, q_scale, k_scale, layout_flag,
                                                   1 if is_causal else 0, 2, sm_scale, 1 if return_lse else 0,
                                                   sparse, smooth_v=smooth_v, exact_exp=exact_exp,
-                                                  two_waves=two_waves)
+                                                  two_waves=two_waves, pv_f16=pv_f16)
         o = o[..., :head_dim_og]
         if return_lse:
             return o, lse / 1.44269504

@@ -100,4 +100,8 @@ __device__ __forceinline__ void buffer_load16_lds(__amdgpu_buffer_rsrc_t rsrc, u
 // The one-wave-per-q-block kernel (D = 64, no lse, no score dump, plain launch).  out_dtype: PARO_DTYPE_*.
 int launch_attn_w64(const AttnParams& p, int out_dtype, bool causal, bool exact, hipStream_t st);
 
+// The kernel with a float16 P.V product (attn_sparse_pv16.hip): p.v8 points at paro_v_f16_pack's tiles, p.v_scale
+// and p.v_mean may be null.  Either head size, with or without lse, plain launch.
+int launch_attn_pv16(const AttnParams& p, int D, int out_dtype, bool causal, hipStream_t st);
+
 }  // namespace paro

@@ -790,11 +790,14 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
                             int64_t k_stride_h, int64_t k_stride_n, int64_t o_stride_b, int64_t o_stride_h,
                             int64_t o_stride_n, float sm_scale, int is_causal, int flags, const int32_t* orders,
                             int n_text, int F, int Hh, int W, void* stream) {
-  PARO_CHECK((flags & ~(PARO_ATTN_EXACT_EXP | PARO_ATTN_PACED | PARO_ATTN_UNPACED | PARO_ATTN_TWO_WAVES)) == 0 &&
+  PARO_CHECK((flags & ~(PARO_ATTN_EXACT_EXP | PARO_ATTN_PACED | PARO_ATTN_UNPACED | PARO_ATTN_TWO_WAVES |
+                        PARO_ATTN_PV_F16)) == 0 &&
                  (flags & (PARO_ATTN_PACED | PARO_ATTN_UNPACED)) != (PARO_ATTN_PACED | PARO_ATTN_UNPACED),
              PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
-  PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && v_scale && sparse && out, PARO_ERR_RUNTIME,
+  const bool pv16 = (flags & PARO_ATTN_PV_F16) != 0;
+  PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && (v_scale || pv16) && sparse && out, PARO_ERR_RUNTIME,
              "paro_attn_sparse_fwd: null tensor pointer");
+  PARO_CHECK(!pv16 || s_dump == nullptr, PARO_ERR_UNSUPPORTED, "the score dump is not available with PARO_ATTN_PV_F16");
   PARO_CHECK(B > 0 && H > 0 && Hkv > 0 && Nq > 0 && Nk > 0, PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: empty shape");
   PARO_CHECK(D == 64 || D == 128, PARO_ERR_INVALID_VALUE, "Unsupported head dim: %d", D);
   PARO_CHECK(H % Hkv == 0, PARO_ERR_INVALID_VALUE, "num_qo_heads (%d) must be divisible by num_kv_heads (%d)", H, Hkv);
@@ -819,7 +822,7 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
              PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: one head of key/value spans 2 GiB or more (kv_len %d, stride %lld)",
              Nk, (long long)k_stride_n);
   // ring stages + the list of kept blocks (6 bytes each) have to fit the 160 KB of LDS of one CU
-  {
+  if (!pv16) {
     const int64_t ring = D == 128 ? 2 * 2 * 64 * 128 : 3 * 2 * 64 * 64;
     PARO_CHECK(ring + ((int64_t)nbk + 8) * 6 + 64 <= 160 * 1024, PARO_ERR_RUNTIME,
                "kv_len %d: the list of %d key blocks does not fit the local data share", Nk, nbk);
@@ -838,6 +841,8 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
   hipStream_t st = (hipStream_t)stream;
   const bool dump = s_dump != nullptr;
   const bool exact = (flags & PARO_ATTN_EXACT_EXP) != 0;
+  // float16 P.V product: a kernel of its own (true exponentials, plain launch)
+  if (pv16) return launch_attn_pv16(p, D, out_dtype, is_causal != 0, st);
   // D = 64 without lse or score dump: one wave per q-block (attn_sparse_w64.hip), unless the caller asks for the
   // two-wave kernel or the launch is to be paced (only the two-wave kernel has the paced form)
   if (D == 64 && lse == nullptr && !dump && (flags & PARO_ATTN_TWO_WAVES) == 0 && !want_pacing(p, D))
@@ -891,6 +896,11 @@ extern "C" int64_t paro_attn_workspace_bytes(int B, int Hkv, int Nk, int D) {
          al(paro_v_fp8_partial_floats(B, Hkv, Nk, D) * 4);
 }
 
+extern "C" int64_t paro_attn_workspace_bytes_for(int B, int Hkv, int Nk, int D, int flags) {
+  if (flags & PARO_ATTN_PV_F16) return (paro_v_f16_bytes(B, Hkv, Nk, D) + 255) & ~(int64_t)255;
+  return paro_attn_workspace_bytes(B, Hkv, Nk, D);
+}
+
 extern "C" int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, const void* v, int v_dtype, void* out,
                                         int out_dtype, const float* q_scale, const float* k_scale,
                                         const uint8_t* sparse, int64_t sparse_batch_stride, float* lse,
@@ -911,9 +921,18 @@ extern "C" int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, cons
              "paro_qk_int8_sv_f16_attn: workspace must be a 256-byte aligned device buffer");
   PARO_CHECK(B > 0 && Hkv > 0 && Nk > 0 && (D == 64 || D == 128), PARO_ERR_INVALID_VALUE,
              "Unsupported shape or head dim: B=%d Hkv=%d Nk=%d D=%d", B, Hkv, Nk, D);
-  PARO_CHECK(workspace_bytes >= paro_attn_workspace_bytes(B, Hkv, Nk, D), PARO_ERR_RUNTIME,
+  PARO_CHECK(workspace_bytes >= paro_attn_workspace_bytes_for(B, Hkv, Nk, D, flags), PARO_ERR_RUNTIME,
              "paro_qk_int8_sv_f16_attn: workspace of %lld bytes is smaller than the %lld needed",
-             (long long)workspace_bytes, (long long)paro_attn_workspace_bytes(B, Hkv, Nk, D));
+             (long long)workspace_bytes, (long long)paro_attn_workspace_bytes_for(B, Hkv, Nk, D, flags));
+  if (flags & PARO_ATTN_PV_F16) {
+    // float16 P.V product: V goes into float16 tiles as it is (no scale, no mean; smooth_v has nothing to act on)
+    int rc = paro_v_f16_pack(v, v_dtype, workspace, B, Hkv, Nk, D, v_stride_b, v_stride_h, v_stride_n, stream);
+    if (rc) return rc;
+    return paro_attn_sparse_fwd(q8, k8, (const uint8_t*)workspace, q_scale, k_scale, nullptr, nullptr, sparse,
+                                sparse_batch_stride, out, out_dtype, lse, nullptr, B, H, Hkv, Nq, Nk, D, q_stride_b,
+                                q_stride_h, q_stride_n, k_stride_b, k_stride_h, k_stride_n, o_stride_b, o_stride_h,
+                                o_stride_n, sm_scale, is_causal, flags, stream);
+  }
   auto al = [](int64_t x) { return (x + 255) & ~(int64_t)255; };
   uint8_t* ws = (uint8_t*)workspace;
   uint8_t* v8 = ws;
