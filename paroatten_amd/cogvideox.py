@@ -92,12 +92,16 @@ SHARED_TABLES = _SharedTables()
 class _ParoProcessorBase:
     """State and helpers shared by the CogVideoX and Wan processors."""
 
-    def __init__(self, grid: Optional[Sequence[int]] = None, smooth_k: bool = False, exact_exp: bool = False):
+    def __init__(self, grid: Optional[Sequence[int]] = None, smooth_k: bool = False, exact_exp: bool = False,
+                 pv_f16: bool = False):
         if not hasattr(F, "scaled_dot_product_attention"):
             raise ImportError("this attention processor requires PyTorch 2.0 or newer")
         self.grid = None if grid is None else tuple(int(x) for x in grid)
         self.smooth_k = smooth_k
         self.exact_exp = exact_exp
+        # accuracy mode of the attention kernel: the float16 P.V product of the reference instead of FP8
+        # (about half the speed; V is then permuted and tiled in float16 by two more passes)
+        self.pv_f16 = pv_f16
         self._timer = _PathTimer()
         self.time_accum = {"total": 0.0}
         self.call_count = 0
@@ -168,15 +172,19 @@ class _ParoProcessorBase:
             query, _, _ = PM.rope_permute(query, None, None, torch.zeros_like(orders), grid, n_text, cos, sin)
             cos = sin = None
         # (smoothing: the mean of the rotated K is taken inside the same call)
-        return PM.rope_permute_quant(query, key, value, orders, grid, n_text, cos, sin,
-                                     km="mean" if self.smooth_k else None)
+        ops = PM.rope_permute_quant(query, key, value, orders, grid, n_text, cos, sin,
+                                    km="mean" if self.smooth_k else None)
+        if self.pv_f16:
+            _, _, vp = PM.rope_permute(None, None, value, orders, grid, n_text)
+            ops = ops._replace(v8=qattn.v_f16_tiles(vp), v_scale=None, v_mean=None)
+        return ops
 
     def _sparse_attention(self, ops, out, sm_scale, orders, grid, n_text):
         """Block-sparse attention on the prepared operands; the inverse permutation (permute_attn_out)
         is part of the kernel's stores, `out` is the [B,H,N,D] view of the token-major result."""
         qattn.attn_sparse_prepacked(ops.q8, ops.k8, ops.v8, ops.v_scale, ops.v_mean, out, ops.q_scale, ops.k_scale,
                                     sm_scale, self._mask(), exact_exp=self.exact_exp,
-                                    unpermute=(orders, grid, n_text))
+                                    unpermute=(orders, grid, n_text), pv_f16=self.pv_f16)
 
     def get_time_stats(self):
         self._timer.fold(block=True)

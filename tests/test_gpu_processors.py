@@ -131,6 +131,25 @@ def test_cogvideox_processor_against_oracle(dev, smooth_k):
 
 
 @torch.no_grad()
+def test_cogvideox_processor_accuracy_mode(dev):
+    """pv_f16=True: the processor's attention runs the float16 P.V product; against the oracle the attention's
+    share of the error drops from FP8's 4 % to what the bfloat16 projections round to."""
+    from paroatten_amd import PARO_CogVideoXAttnProcessor2_0
+    attn, hidden, text, rotary, masks, plan, grid, n_text = _cog_case(dev)
+    ref_h, ref_t, *_ = _cog_expected(attn, hidden, text, rotary, masks[1, 1], plan, 1, grid, n_text, True)
+    rms = {}
+    for pv16 in (False, True):
+        proc = PARO_CogVideoXAttnProcessor2_0(grid=grid, smooth_k=True, pv_f16=pv16)
+        proc.permute_plan, proc.i_block, proc.i_timestep = plan, 1, 1
+        proc.sparse_mask = masks.to(dev)
+        out_h, out_t = proc(attn, hidden, text, image_rotary_emb=(rotary[0].to(dev), rotary[1].to(dev)))
+        rms[pv16] = max(_rel_rms(out_h, ref_h), _rel_rms(out_t, ref_t))
+        assert cosine(out_h.cpu(), ref_h.cpu()) >= (0.9999 if pv16 else 0.999)
+    assert rms[True] <= 0.012, rms           # bfloat16 rounding of the attention output and of the projection
+    assert rms[True] < 0.5 * rms[False], rms
+
+
+@torch.no_grad()
 def test_cogvideox_processor_prefetch_equals_resident_mask(dev):
     from paroatten_amd import PARO_CogVideoXAttnProcessor2_0
     from paroatten_amd.prefetch_utils import SparseMaskPrefetchStream
