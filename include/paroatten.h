@@ -59,7 +59,7 @@ extern "C" {
                                  only; about half the speed of the default (the matrix pipe runs float16 at half the
                                  FP8 rate). */
 
-/* Version of this ABI (bumped when a signature changes). */
+/* Version of this ABI (bumped when a signature changes or an export leaves the library; currently 2). */
 int paro_abi_version(void);
 /* Message of the last error on this thread ("" if none). Host pointer, valid until the next call. */
 const char* paro_last_error(void);

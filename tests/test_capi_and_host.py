@@ -26,10 +26,10 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), f"{n} declared in include/paroatten.h but not exported"
         assert n in L.SIGNATURES, f"{n} has no ctypes signature"
     assert set(L.SIGNATURES) == set(names)
-    assert lib.paro_abi_version() == 1
+    assert lib.paro_abi_version() == 2
     assert lib.paro_build_arch() == b"gfx950"
     raw = ctypes.CDLL(str(L.LIB_PATH))
-    assert raw.paro_abi_version() == 1
+    assert raw.paro_abi_version() == 2
 
 
 def test_measurement_aids_live_outside_the_product_library():
