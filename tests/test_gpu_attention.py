@@ -301,8 +301,8 @@ def test_fast_path_overflow_of_a_single_row(dev, D, row):
 def test_paced_launch_is_bit_identical(dev, D, H, N, monkeypatch):
     """PARO_ATTN_PACED (resident workgroups per XCD that take their q-blocks generation by generation)
     against PARO_ATTN_UNPACED: the launch form may not change a single bit, whether the workgroups wait
-    for each other (default) or never do (a spin limit of zero, forced through the environment: the
-    meeting point only paces).  Shapes with more q-blocks per XCD than workgroups fit on it, so that the
+    for each other (default: for all but a share of the generation), for all, for next to none, or never
+    (a spin limit of zero, forced through the environment: the meeting point only paces).  Shapes with more q-blocks per XCD than workgroups fit on it, so that the
     paced kernel really runs several generations; checked against the oracle on one head."""
     from paroatten_amd import _qattn_sm80 as qattn
     from paroatten_amd import quant as Q
@@ -314,11 +314,15 @@ def test_paced_launch_is_bit_identical(dev, D, H, N, monkeypatch):
     q8, qs, k8, ks = Q.per_warp_int8(q, k, None, BLKQ=64, WARPQ=32, BLKK=64)
     v8, vsc, vm = Q.per_channel_fp8(v)
     outs = []
-    for pacing, spins in ((False, None), (True, None), (True, "0"), (True, "3")):
-        if spins is None:
-            monkeypatch.delenv("PARO_ATTN_PACE_SPINS", raising=False)
-        else:
-            monkeypatch.setenv("PARO_ATTN_PACE_SPINS", spins)
+    # (spin limit, arrivals a generation does not wait for): the library's defaults, no waiting at all, a short
+    # limit, waiting for every workgroup, waiting for next to none
+    for pacing, spins, slack in ((False, None, None), (True, None, None), (True, "0", None), (True, "3", None),
+                                 (True, None, "0"), (True, None, "100000"), (True, "5", "7")):
+        for name, val in (("PARO_ATTN_PACE_SPINS", spins), ("PARO_ATTN_PACE_SLACK", slack)):
+            if val is None:
+                monkeypatch.delenv(name, raising=False)
+            else:
+                monkeypatch.setenv(name, val)
         out = torch.full_like(q, float("nan"))
         lse = qattn.attn_sparse_prepacked(q8, k8, v8, vsc, vm, out, qs, ks, D ** -0.5, mask, return_lse=1, pacing=pacing)
         outs.append((out, lse))
