@@ -12,6 +12,7 @@
 // guard: paroattention/core.py:168-174 works around it) every call runs under a guard for the tensors'
 // device and on torch's current stream of that device.
 #include <torch/extension.h>
+#include <atomic>
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
@@ -62,6 +63,13 @@ Layout layout_of(const torch::Tensor& x, int tensor_layout) {
 }
 
 // ---- _qattn_sm80 ------------------------------------------------------------------------------------
+// The reference's positional signature has no room for this library's attention flags (PARO_ATTN_* of
+// include/paroatten.h: exact exponentials, the float16 P.V product, launch forms).  A process-wide default,
+// set_attention_flags(), lets a caller of the compiled module choose them; 0 = the library's defaults.
+static std::atomic<int> g_attention_flags{0};
+void set_attention_flags(int flags) { g_attention_flags.store(flags); }
+int get_attention_flags() { return g_attention_flags.load(); }
+
 torch::Tensor qk_int8_sv_f16_accum_f16_attn(torch::Tensor query, torch::Tensor key, torch::Tensor value,
                                             torch::Tensor output, torch::Tensor query_scale,
                                             torch::Tensor key_scale, int tensor_layout, int is_causal,
@@ -120,7 +128,8 @@ torch::Tensor qk_int8_sv_f16_accum_f16_attn(torch::Tensor query, torch::Tensor k
   const c10::DeviceGuard guard(query.device());
   torch::Tensor lse = torch::empty({0});
   if (return_lse) lse = torch::empty({B, H, Nq}, query.options().dtype(at::kFloat));
-  const int64_t ws_bytes = paro_attn_workspace_bytes((int)B, (int)Hkv, (int)Nk, (int)D);
+  const int flags = g_attention_flags.load();
+  const int64_t ws_bytes = paro_attn_workspace_bytes_for((int)B, (int)Hkv, (int)Nk, (int)D, flags);
   torch::Tensor ws = torch::empty({ws_bytes}, query.options().dtype(at::kByte));
   check_rc(paro_qk_int8_sv_f16_attn(
       query.data_ptr<int8_t>(), key.data_ptr<int8_t>(), value.data_ptr(), half_code(value, "qk_int8_sv_f16_accum_f16_attn"),
@@ -129,7 +138,7 @@ torch::Tensor qk_int8_sv_f16_accum_f16_attn(torch::Tensor query, torch::Tensor k
       ws.data_ptr(), ws_bytes, (int)B, (int)H, (int)Hkv, (int)Nq, (int)Nk, (int)D, query.stride(0), query.stride(sh),
       query.stride(sn), key.stride(0), key.stride(sh), key.stride(sn), value.stride(0), value.stride(sh), value.stride(sn),
       output.stride(0), output.stride(sh), output.stride(sn), tensor_layout, is_causal, qk_quant_gran, sm_scale,
-      /*smooth_v=*/1, /*flags=*/0, stream_of(query)));
+      /*smooth_v=*/1, flags, stream_of(query)));
   return lse;
 }
 
@@ -308,6 +317,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("abi_version", &paro_abi_version);
   auto qattn = m.def_submodule("_qattn_sm80");
   qattn.def("qk_int8_sv_f16_accum_f16_attn", &qk_int8_sv_f16_accum_f16_attn, "QK int8 sv f16 accum f16 attn");
+  qattn.def("set_attention_flags", &set_attention_flags,
+            "process-wide PARO_ATTN_* flags of the attention entry point (1 exact exponentials, 16 float16 P.V product, ...)");
+  qattn.def("get_attention_flags", &get_attention_flags);
   qattn.def("qk_int4_sv_f16_accum_f16_attn", &prototype_variant);
   qattn.def("qk_int4_sv_int8_accum_f16_attn", &prototype_variant);
   qattn.def("qk_int8_sv_int8_accum_f16_attn", &prototype_variant);

@@ -90,6 +90,18 @@ def test_extension_matches_ctypes_mirrors_bit_for_bit(ext, dev):
         assert res[0][1].shape == res[1][1].shape and torch.equal(res[0][1].cpu(), res[1][1].cpu())
         if not lse_on:
             assert res[0][1].numel() == 0 and not res[0][1].is_cuda     # the reference returns an empty CPU tensor
+    # the flags the positional signature has no room for: a process-wide default of the compiled module
+    from paroatten_amd import _lib
+    assert ext._qattn_sm80.get_attention_flags() == 0
+    for flags, kw in ((_lib.PARO_ATTN_PV_F16, dict(pv_f16=True)), (_lib.PARO_ATTN_EXACT_EXP, dict(exact_exp=True))):
+        ext._qattn_sm80.set_attention_flags(flags)
+        try:
+            a, b = torch.empty_like(q), torch.empty_like(q)
+            ext._qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, a, qs, ks, 1, 0, 2, D ** -0.5, 0, mask)
+        finally:
+            ext._qattn_sm80.set_attention_flags(0)
+        _qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, b, qs, ks, 1, 0, 2, D ** -0.5, 0, mask, **kw)
+        assert torch.equal(a, b), flags
     with pytest.raises(ValueError, match="tensor_layout must be 0 or 1"):
         ext._qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, torch.empty_like(q), qs, ks, 7, 0, 2, 0.125, 0, mask)
     with pytest.raises(RuntimeError, match="Tensor sparse must have shape"):
