@@ -208,11 +208,19 @@ __global__ void __launch_bounds__(128, 2) attn_sparse_pv16_kernel(const AttnPara
     }
 
     // -- running maximum, refreshed only when a weight would exceed 2^(OFFSET + HEADROOM)
-    float smax = s[0][0];
+    // (four interleaved v_max3 chains; the values are integers read as floats: no NaN to canonicalise)
+    float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[0][8], s[0][9], s[0][10]);
+    float mx2 = max3(s[1][0], s[1][1], s[1][2]), mx3 = max3(s[1][8], s[1][9], s[1][10]);
 #pragma unroll
-    for (int mt = 0; mt < 2; mt++)
-#pragma unroll
-      for (int i = 0; i < 16; i++) smax = fmaxf(smax, s[mt][i]);
+    for (int i = 3; i < 7; i += 2) {
+      mx0 = max3(mx0, s[0][i], s[0][i + 1]);
+      mx1 = max3(mx1, s[0][i + 8], s[0][i + 9]);
+      mx2 = max3(mx2, s[1][i], s[1][i + 1]);
+      mx3 = max3(mx3, s[1][i + 8], s[1][i + 9]);
+    }
+    mx0 = max3(mx0, s[0][7], s[0][15]);
+    mx2 = max3(mx2, s[1][7], s[1][15]);
+    const float smax = max3(max3(mx0, mx1, mx2), mx3, mx3);
     const float m_blk = fmaf(partner_max(smax), c, -S_MAGIC_F * c);
     if (__ballot(m_blk > m_thr) != 0ull) {
       const float m_new = fmaxf(m_i, m_blk);
