@@ -45,8 +45,10 @@ extern "C" {
 #define PARO_ATTN_UNPACED 4   /* one workgroup per q-block, started as the hardware pleases.  With neither flag the
                                  library paces when one head's K8 + V8 exceed an XCD's 4 MB L2 (environment variable
                                  PARO_ATTN_PACING=0/1 overrides that default).  Scattered masks on long sequences gain
-                                 (Wan 720p, uniformly random blocks: 26 -> 35 % of the MFMA peak, 3.3x fewer L2 fills);
-                                 masks made of one contiguous run per row lose a few per cent. */
+                                 (Wan 720p, uniformly random blocks: 26 -> 39 % of the MFMA peak, 4x fewer L2 fills);
+                                 masks made of one contiguous run per row lose a few per cent.  A generation waits for
+                                 all but a share of its workgroups (PARO_ATTN_PACE_SLACK; default half the L2's share
+                                 of a head, at most a quarter of them) and at most PARO_ATTN_PACE_SPINS rounds. */
 #define PARO_ATTN_TWO_WAVES 8 /* kernel form, results are bit-identical either way: two waves per 64-row q-block
                                  (32 q-rows each) also where the library would pick the one-wave-per-q-block
                                  kernel (head size 64, no lse, plain launch), which is the faster of the two there */
