@@ -53,9 +53,9 @@ WORKLOAD_DENSITIES = {
 # CogVideoX: the same at every density (one head's K8 + V8 stay in the L2).  Wan: L2 fills, with the paced
 # launch; they vary by tens of percent from box to box at 720p, where a head is five times the L2.
 ATTN_TRAFFIC_BYTES = {
-    "cogvideox5b": int((169381 * 2.0 + 213315 * 1.0) * 1024),
-    "wan14b_480p": int((1218830 * 2.0 + 335512 * 1.0) * 1024),
-    "wan14b_720p": int((16747800 * 2.0 + 813568 * 1.0) * 1024),
+    "cogvideox5b": int((169346 * 2.0 + 213315 * 1.0) * 1024),
+    "wan14b_480p": int((1142630 * 2.0 + 335455 * 1.0) * 1024),
+    "wan14b_720p": int((16238000 * 2.0 + 812113 * 1.0) * 1024),
 }
 
 
