@@ -12,7 +12,7 @@ from . import _lib
 
 _lib.load()  # fail at import time if libparoatten_hip.so is missing: there is no fallback path
 
-from . import _fused, _qattn_sm80, _rope, cogvideox, core, permute, plans, prefetch_utils, quant, wan  # noqa: E402
+from . import _fused, _qattn_sm80, _rope, cogvideox, core, permute, plans, prefetch_utils, quant, utils, wan  # noqa: E402
 from .cogvideox import PARO_CogVideoXAttnProcessor, PARO_CogVideoXAttnProcessor2_0  # noqa: E402
 from .core import paroattn, paroattn_qk_int8_pv_fp16_cuda  # noqa: E402
 from .wan import PARO_WanAttnProcessor, PARO_WanAttnProcessor2_0, set_paro_processors  # noqa: E402

@@ -237,7 +237,7 @@ def test_import_paroattention_resolves_by_itself():
         "import paroattention, paroatten_amd\n"
         "assert paroattention is paroatten_amd\n"
         "import paroattention.core, paroattention.quant, paroattention.cogvideox, paroattention.wan\n"
-        "import paroattention.prefetch_utils, paroattention.prefetch_wan\n"
+        "import paroattention.prefetch_utils, paroattention.prefetch_wan, paroattention.utils\n"
         "import paroattention._qattn_sm80, paroattention._fused, paroattention._rope\n"
         "from paroattention import paroattn, paroattn_qk_int8_pv_fp16_cuda, PARO_CogVideoXAttnProcessor2_0, "
         "PARO_WanAttnProcessor2_0\n"

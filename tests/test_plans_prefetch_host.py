@@ -70,6 +70,23 @@ def test_timestep_callback_writes_every_processor(blocks_attr):
     assert cb.timestep_history[0]["step"] == 5 and cb.timestep_history[0]["timestep"] == 801.0
 
 
+def test_utils_timestep_callback_keeps_its_own_convention():
+    """paroattention/utils.py:13-34: the transformer gets (step + 1) / total as a float, the processors the
+    index int(that * T); worked by hand for step 5 of 20, T = 10: 0.3 and 3; step 25 is not wrapped: 1.3, 13"""
+    from paroatten_amd import utils
+    procs = [types.SimpleNamespace(i_timestep=-5) for _ in range(2)]
+    blocks = [types.SimpleNamespace(attn1=types.SimpleNamespace(processor=p)) for p in procs]
+    transformer = types.SimpleNamespace(transformer_blocks=blocks)
+    pipe = types.SimpleNamespace(transformer=transformer, scheduler=types.SimpleNamespace(timesteps=list(range(20))))
+    cb = utils.TimestepCallback(num_timestep_for_sparse_mask=10)
+    kw = {"latents": None}
+    assert cb.on_step_end(pipe, 5, 801, kw) is kw
+    assert transformer.i_timestep == pytest.approx(0.3) and all(p.i_timestep == 3 for p in procs)
+    cb.on_step_end(pipe, 25, 1, kw)
+    assert transformer.i_timestep == pytest.approx(1.3) and all(p.i_timestep == 13 for p in procs)
+    assert [h["step"] for h in cb.timestep_history] == [5, 25]
+
+
 @pytest.mark.parametrize("n", [1, 7, 8, 9, 127, 128, 1000])
 def test_pack_mask_bits_matches_numpy(n):
     g = torch.Generator().manual_seed(n)
