@@ -22,6 +22,13 @@ __all__ = ["paroattn", "paroattn_qk_int8_pv_fp16_cuda", "PARO_CogVideoXAttnProce
            "set_paro_processors", "install_alias", "compiled_extension"]
 
 
+def __getattr__(name):
+    # the two names of paroattention/__init__.py:4-5 that need diffusers: resolved on first use
+    if name in ("PARO_WanTransformerBlock", "PARO_WanTransformer3DModel"):
+        return wan.diffusers_wan_classes()[name]
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+
+
 def compiled_extension():
     """The PyTorch-ROCm C++ extension (csrc/torch_binding.cpp -> paroatten_amd/_ext.so): submodules
     `_qattn_sm80`, `_fused`, `_rope` with the reference's positional pybind signatures, bound to the same

@@ -157,3 +157,44 @@ def set_paro_processors(transformer, permute_plan, sparse_mask=None, prefetch_st
             block.attn1.processor = p
         procs.append(p)
     return procs
+
+
+_DIFFUSERS_WAN = {}
+
+
+def diffusers_wan_classes():
+    """`PARO_WanTransformerBlock` and `PARO_WanTransformer3DModel` (paroattention/wan.py:525-783): in the reference
+    these are copies of diffusers' Wan transformer whose only change is the processor of `attn1` (wan.py:550).
+    Here they are SUBCLASSES of the installed diffusers classes, built on first use: the block installs a
+    `PARO_WanAttnProcessor2_0` on its `attn1`, the model builds its blocks from that class, everything else
+    (weights, config, `from_pretrained`, forward) is diffusers' own.  Raises ImportError without diffusers."""
+    if _DIFFUSERS_WAN:
+        return _DIFFUSERS_WAN
+    try:
+        from diffusers.models.transformers import transformer_wan as tw
+    except Exception as e:
+        raise ImportError("PARO_WanTransformer3DModel / PARO_WanTransformerBlock subclass diffusers' Wan transformer, "
+                          f"and diffusers is not importable here ({e}); on an existing model use "
+                          "paroatten_amd.set_paro_processors(model, permute_plan, ...)") from e
+
+    class PARO_WanTransformerBlock(tw.WanTransformerBlock):
+        def __init__(self, *args, **kwargs):
+            super().__init__(*args, **kwargs)
+            self.attn1.set_processor(PARO_WanAttnProcessor2_0())
+
+    class PARO_WanTransformer3DModel(tw.WanTransformer3DModel):
+        def __init__(self, *args, **kwargs):
+            super().__init__(*args, **kwargs)
+            # (the blocks exist by now; their projections and norms are what the processor drives)
+            for block in self.blocks:
+                block.attn1.set_processor(PARO_WanAttnProcessor2_0())
+
+    _DIFFUSERS_WAN.update(PARO_WanTransformerBlock=PARO_WanTransformerBlock,
+                          PARO_WanTransformer3DModel=PARO_WanTransformer3DModel)
+    return _DIFFUSERS_WAN
+
+
+def __getattr__(name):
+    if name in ("PARO_WanTransformerBlock", "PARO_WanTransformer3DModel"):
+        return diffusers_wan_classes()[name]
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

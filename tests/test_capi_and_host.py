@@ -249,3 +249,46 @@ def test_import_paroattention_resolves_by_itself():
         "print('ok')\n")
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr[-2000:]
+
+
+def test_wan_model_names_subclass_diffusers_when_it_is_there():
+    """paroattention/__init__.py:4-5 exports PARO_WanTransformerBlock and PARO_WanTransformer3DModel; here they are
+    subclasses of diffusers' classes built on first use.  With a stand-in `diffusers` (two classes of the same
+    names and shape: a block with `attn1.set_processor`, a model with `.blocks`) every attn1 ends up with a
+    PARO_WanAttnProcessor2_0; without diffusers the names raise ImportError that names the alternative."""
+    import subprocess
+    import sys
+    code = (
+        "import sys, types\n"
+        "import paroattention\n"
+        "try:\n"
+        "    paroattention.PARO_WanTransformer3DModel\n"
+        "    raise SystemExit('expected ImportError')\n"
+        "except ImportError as e:\n"
+        "    assert 'set_paro_processors' in str(e)\n"
+        "class Attn:\n"
+        "    def __init__(self): self.processor = 'stock'\n"
+        "    def set_processor(self, p): self.processor = p\n"
+        "class WanTransformerBlock:\n"
+        "    def __init__(self, dim=8): self.dim = dim; self.attn1 = Attn(); self.attn2 = Attn()\n"
+        "class WanTransformer3DModel:\n"
+        "    def __init__(self, num_layers=3): self.blocks = [WanTransformerBlock() for _ in range(num_layers)]\n"
+        "tw = types.ModuleType('diffusers.models.transformers.transformer_wan')\n"
+        "tw.WanTransformerBlock, tw.WanTransformer3DModel = WanTransformerBlock, WanTransformer3DModel\n"
+        "for name in ('diffusers', 'diffusers.models', 'diffusers.models.transformers'):\n"
+        "    m = types.ModuleType(name); m.__path__ = []; sys.modules[name] = m\n"
+        "sys.modules['diffusers.models.transformers.transformer_wan'] = tw\n"
+        "sys.modules['diffusers.models.transformers'].transformer_wan = tw\n"
+        "from paroattention import PARO_WanTransformer3DModel, PARO_WanTransformerBlock, PARO_WanAttnProcessor2_0\n"
+        "from paroattention.wan import PARO_WanTransformer3DModel as M2\n"
+        "assert M2 is PARO_WanTransformer3DModel and issubclass(PARO_WanTransformer3DModel, WanTransformer3DModel)\n"
+        "model = PARO_WanTransformer3DModel(num_layers=4)\n"
+        "assert len(model.blocks) == 4\n"
+        "assert all(isinstance(b.attn1.processor, PARO_WanAttnProcessor2_0) for b in model.blocks)\n"
+        "assert all(b.attn2.processor == 'stock' for b in model.blocks)\n"
+        "assert len({id(b.attn1.processor) for b in model.blocks}) == 4\n"
+        "blk = PARO_WanTransformerBlock(dim=16)\n"
+        "assert blk.dim == 16 and isinstance(blk.attn1.processor, PARO_WanAttnProcessor2_0)\n"
+        "print('ok')\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr[-2000:]
