@@ -61,6 +61,13 @@ extern "C" {
                                  only; about half the speed of the default (the matrix pipe runs float16 at half the
                                  FP8 rate). */
 
+#define PARO_ATTN_QK_PER_THREAD 32 /* q_scale / k_scale have the reference's per-thread granularity (qk_quant_gran 3,
+                                 csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133, shapes :1034-1038): q_scale
+                                 [B,H,nbq*2*8], scale g of a 32-row group for its rows r with r % 8 == g; k_scale
+                                 [B,Hkv,nbk*4] (16-byte aligned), scale j of a 64-key block for its keys c with
+                                 (c % 8) / 2 == j.  Two-wave kernel with true exponentials, plain launch; with
+                                 neither PARO_ATTN_PV_F16 nor s_dump.  paro_quant_int8_per_thread makes such scales. */
+
 /* Version of this ABI (bumped when a signature changes or an export leaves the library; currently 2). */
 int paro_abi_version(void);
 /* Message of the last error on this thread ("" if none). Host pointer, valid until the next call. */
@@ -88,6 +95,22 @@ int paro_quant_int8(const void* x, int dtype, const void* mean, int8_t* out, flo
                     int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n,
                     int64_t scale_stride_b, int64_t scale_stride_h,
                     int group, int n_groups, int has_sm_scale, float sm_scale, void* stream);
+
+/* (1') The same arithmetic with the per-thread grouping of qk_quant_gran 3.  The reference declares that
+ * granularity in its attention kernel (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133) and checks the
+ * scale shapes (:1034-1038) but ships no quantiser for it (paroattention/core.py:204-205 calls the per-block
+ * one, whose scales that check rejects); the grouping is the one the kernel's indexing implies.
+ *   is_key == 0 (Q): eight scales per 32 tokens; group g of tokens 32 w + g + 8 j, j = 0..3;
+ *                    scale [B,H, ceil(N/64)*2*8] at (w * 8 + g)
+ *   is_key == 1 (K): four scales per 64 tokens; group j of tokens 64 w + 8 t + 2 j + e, t = 0..7, e = 0..1;
+ *                    scale [B,H, ceil(N/64)*4] at (w * 4 + j)
+ * Tokens >= N read as 0; groups that lie wholly past N get scale 1e-7 / 127.  scale contiguous. */
+int paro_quant_int8_per_thread(const void* x, int dtype, const void* mean, int8_t* out, float* scale,
+                               int B, int H, int N, int D,
+                               int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_n,
+                               int64_t mean_stride_b, int64_t mean_stride_h,
+                               int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_n,
+                               int is_key, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * (2a) V -> FP8 (e4m3fn) with per-(b,h,channel) mean smoothing and scale, written in the
@@ -186,7 +209,7 @@ int paro_attn_sparse_unpermute_fwd(const int8_t* q8, const int8_t* k8, const uin
  * (2c) The reference's extension entry point in one call: V (fp16/bf16) -> FP8 tiles, then (2b).
  * Stands in for qk_int8_sv_f16_accum_f16_attn as bound at csrc/qattn/pybind_sm80.cpp:23 /
  * csrc/qattn/attn_cuda_sm80.h:19-31: same tensors, same integer flags (tensor_layout 0 = NHD,
- * 1 = HND; qk_quant_gran 2 = per_warp, 3 = per_thread -> PARO_ERR_UNSUPPORTED), same checks.
+ * 1 = HND; qk_quant_gran 2 = per_warp, 3 = per_thread: PARO_ATTN_QK_PER_THREAD is set), same checks.
  * workspace: paro_attn_workspace_bytes() bytes of device memory (256-byte aligned).
  * ------------------------------------------------------------------------------------------- */
 int64_t paro_attn_workspace_bytes(int B, int Hkv, int Nk, int D);

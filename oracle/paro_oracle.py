@@ -12,9 +12,14 @@ forms, brute force on tiny inputs, reduction to a library routine) in tests/test
 Pinning status
   quant_int8 / per_warp_int8 / per_block_int8 : pinned (closed-form KAT of bench/test.py,
         invariants, brute force)
+  per_thread_scale_index / per_thread_int8    : pinned (the index law against an enumeration of the
+        reference kernel's accumulator lanes, :112-116 and :129-133 of its .cu; the quantiser reduces to
+        quant_int8 on tokens regrouped so that every group is contiguous)
   qk_int32                                    : pinned (int64 einsum brute force)
   sparse_attention                            : pinned (reduces to softmax(mask)@V library
-        routine, dense SDPA special case, empty-row and K-smoothing invariants, lse closed form)
+        routine, dense SDPA special case, empty-row and K-smoothing invariants, lse closed form; with
+        per-thread scales: reduces to the per-warp result for scales that are constant per group, and to
+        fp64 softmax attention on tensors dequantised row by row)
   permute maps / permute_qk / permute_attn_out: pinned (torch.permute library routine, the
         reference's literal tables, inverse∘forward = id)
   rope_wan                                    : pinned (complex rotation, norm, composition)
@@ -110,6 +115,52 @@ def per_warp_int8(q, k, km=None, BLKQ=128, WARPQ=32, BLKK=64):
     return q8, qs, k8, ks
 
 
+def per_thread_scale_index(n: int, is_key: bool) -> torch.Tensor:
+    """Scale index of each of n tokens at the per-thread granularity (qk_quant_gran 3) of
+    qk_int_sv_f16_attn_kernel with CTA_Q = CTA_K = WARP_K = 64, WARP_Q = 32.  A thread of the m16n8
+    accumulator tiles holds rows lane/4 and lane/4 + 8 of every 16-row tile and columns 2*(lane%4),
+    2*(lane%4)+1 of every 8-column tile, and reads q scale `warp*8 + lane/4` and k scale
+    `block*4 + lane%4` (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133).  So query token r uses
+    scale (r//32)*8 + r%8 and key token c uses scale (c//64)*4 + (c%8)//2."""
+    t = torch.arange(n)
+    if is_key:
+        return (t // 64) * 4 + (t % 8) // 2
+    return (t // 32) * 8 + t % 8
+
+
+def quant_int8_per_thread(x: torch.Tensor, is_key: bool, mean: Optional[torch.Tensor] = None):
+    """The arithmetic of quant_int8 on the token groups of per_thread_scale_index.  The reference has no
+    quantiser of this granularity (paroattention/core.py:204-205 calls the per-block one, whose scales the
+    kernel's shape check :1034-1038 rejects): this is the quantiser its kernel's indexing implies.
+    Returns (int8 [B,H,N,D], scale [B,H,ceil(N/64)*(4 if is_key else 16)])."""
+    B, H, N, D = x.shape
+    xf = x.to(torch.float32)
+    if mean is not None:
+        xf = xf - mean.to(torch.float32).reshape(B, H, 1, D)
+    npad = (N + 63) // 64 * 64
+    if npad > N:
+        xf = torch.nn.functional.pad(xf, (0, 0, 0, npad - N))   # tokens >= N read as 0, whatever the mean
+    idx = per_thread_scale_index(npad, is_key)
+    n_scales = npad // 64 * (4 if is_key else 16)
+    tok_amax = xf.abs().amax(dim=-1)
+    amax = torch.zeros(B, H, n_scales, dtype=torch.float32)
+    amax = amax.scatter_reduce(2, idx.expand(B, H, npad), tok_amax, reduce="amax", include_self=True)
+    amax = amax.clamp_min(torch.tensor(1e-7, dtype=torch.float32))
+    scale = amax / torch.tensor(127.0, dtype=torch.float32)
+    inv = torch.tensor(127.0, dtype=torch.float32) / amax
+    q = torch.round(xf * inv[:, :, idx].unsqueeze(-1)).clamp_(-128, 127).to(torch.int8)
+    return q[:, :, :N].contiguous(), scale
+
+
+def per_thread_int8(q, k, km=None):
+    """Q and K at the per-thread granularity (HND); km as in per_warp_int8."""
+    if km is not None:
+        km = km.reshape(k.shape[0], k.shape[1], k.shape[3])
+    q8, qs = quant_int8_per_thread(q, False)
+    k8, ks = quant_int8_per_thread(k, True, mean=km)
+    return q8, qs, k8, ks
+
+
 def per_block_int8(q, k, km=None, BLKQ=128, BLKK=64, sm_scale=None):
     """paroattention/quant.py:22-103 (HND): folds sm_scale*1.44269504 into Q (:91-96)."""
     D = q.shape[-1]
@@ -160,8 +211,10 @@ def sparse_attention(
     out_dtype: torch.dtype = torch.float16,
     compute_dtype: torch.dtype = torch.float32,
     q_chunk: int = 2048,
+    per_thread: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Intended semantics of qk_int8_sv_f16_accum_f16_attn (HND, gran = per_warp):
+    """Intended semantics of qk_int8_sv_f16_accum_f16_attn (HND, gran = per_warp; with per_thread=True
+    gran = per_thread: the scales of row i and column j are those of per_thread_scale_index):
 
       s_ij = (sum_d q8_id k8_jd) * q_scale[b,h,i//warp_q] * k_scale[b,hk,j//blk_k] * sm_scale
       J(i) = { j < N : mask[b,h,i//64,j//64] }  (and j <= i if causal)
@@ -186,13 +239,16 @@ def sparse_attention(
         for h in range(H):
             hk = h // groups
             kf = k8[b, hk].to(compute_dtype)
-            ksc = k_scale[b, hk].to(compute_dtype).repeat_interleave(blk_k)[:Nk]
+            if per_thread:
+                ksc = k_scale[b, hk].to(compute_dtype)[per_thread_scale_index(Nk, True)]
+            else:
+                ksc = k_scale[b, hk].to(compute_dtype).repeat_interleave(blk_k)[:Nk]
             for i0 in range(0, N, q_chunk):
                 i1 = min(N, i0 + q_chunk)
                 qf = q8[b, h, i0:i1].to(compute_dtype)
                 s = qf @ kf.T  # exact integers (< 2^24) in fp32/fp64
                 row = torch.arange(i0, i1)
-                qsc = q_scale[b, h].to(compute_dtype)[row // warp_q]
+                qsc = q_scale[b, h].to(compute_dtype)[per_thread_scale_index(N, False)[row] if per_thread else row // warp_q]
                 s = s * (qsc[:, None] * ksc[None, :]) * sm_scale
                 keep = mask[b, h][row // 64][:, col // 64]
                 if is_causal:

@@ -24,6 +24,7 @@ PARO_ATTN_PACED = 2
 PARO_ATTN_UNPACED = 4
 PARO_ATTN_TWO_WAVES = 8
 PARO_ATTN_PV_F16 = 16
+PARO_ATTN_QK_PER_THREAD = 32
 
 DTYPE_CODE = {torch.float16: 0, torch.bfloat16: 1}
 
@@ -38,6 +39,8 @@ SIGNATURES = {
     "paro_build_arch": (c_char_p, []),
     "paro_quant_int8": (c_int, [_P, _I, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L,
                                 _I, _I, _I, _F, _P]),
+    "paro_quant_int8_per_thread": (c_int, [_P, _I, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _L,
+                                           _I, _P]),
     "paro_v_fp8_bytes": (c_int64, [_I, _I, _I, _I]),
     "paro_v_fp8_partial_floats": (c_int64, [_I, _I, _I, _I]),
     "paro_v_fp8_pack": (c_int, [_P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _I, _P]),

@@ -14,6 +14,9 @@ Differences, all relaxations or added checks:
   * keyword `pv_f16=True` is the accuracy mode (PARO_ATTN_PV_F16): the P.V product in float16 with fp32
     accumulation, as the reference's kernel of this name computes it, instead of FP8 e4m3 P and V: true
     exponentials, V as given (smooth_v has nothing to act on); about half the speed;
+  * `qk_quant_gran=3` (per thread: eight q scales per 32 rows, four k scales per 64 keys, indexed as
+    csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133) runs the two-wave kernel with true exponentials;
+    quant.per_thread_int8 makes such scales (the reference has no quantiser for them);
   * keyword `pacing=True/False` picks the launch form of the attention kernel (see PARO_ATTN_PACED in
     include/paroatten.h; bit-identical results), None leaves it to the library;
   * `sparse` IS validated (the reference reads it through a raw pointer unchecked): bool or uint8,
@@ -120,6 +123,13 @@ def qk_int8_sv_f16_accum_f16_attn(query, key, value, output, query_scale, key_sc
              "Tensor query_scale must have shape (batch_size, num_qo_heads, div_ceil(qo_len, CTA_Q) * (CTA_Q / WARP_Q))")
         _chk(tuple(key_scale.shape) == (B, Hkv, nbk),
              "Tensor key_scale must have shape (batch_size, num_kv_heads, div_ceil(kv_len, CTA_K) * (CTA_K / WARP_K))")
+    else:   # per thread (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:1034-1038)
+        _chk(tuple(query_scale.shape) == (B, H, nbq * 2 * 8),
+             "Tensor query_scale must have shape (batch_size, num_qo_heads, div_ceil(qo_len, CTA_Q) * (CTA_Q / WARP_Q) * 8)")
+        _chk(tuple(key_scale.shape) == (B, Hkv, nbk * 4),
+             "Tensor key_scale must have shape (batch_size, num_kv_heads, div_ceil(kv_len, CTA_K) * (CTA_K / WARP_K) * 4)")
+        if pv_f16:
+            raise NotImplementedError("qk_quant_gran 3 (per thread) is not available with pv_f16")
     # the mask: checked here, unlike the reference
     _chk(sparse.is_cuda, "Tensor sparse must be on CUDA")
     _chk(sparse.dtype in (torch.bool, torch.uint8), "Tensor sparse must have dtype (torch::kBool)")

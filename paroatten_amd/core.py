@@ -12,6 +12,7 @@ from typing import Any, Optional
 import torch
 
 from . import _qattn_sm80 as qattn
+from .quant import per_thread_int8
 from .quant import per_warp_int8 as per_warp_int8_cuda
 
 
@@ -54,10 +55,8 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
     assert qk_quant_gran in ["per_warp", "per_thread"], "qk_quant_gran must be either 'per_warp' or 'per_thread'."
     assert q.device == k.device == v.device, "All tensors must be on the same device."
     assert q.dtype == k.dtype == v.dtype, "All tensors must have the same dtype."
-    if qk_quant_gran == "per_thread":
-        # core.py:204-205 of the reference pairs per-block scales (softmax scale folded in) with
-        # the per-thread kernel path, whose shape check rejects them: it cannot run there either
-        raise NotImplementedError("qk_quant_gran='per_thread' is not implemented; use 'per_warp'")
+    if qk_quant_gran == "per_thread" and pv_f16:
+        raise NotImplementedError("qk_quant_gran='per_thread' is not available with pv_f16")
 
     # launch on the tensors' device, as the reference's set_device workaround does (core.py:168-174)
     with torch.cuda.device(v.device):
@@ -80,11 +79,17 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
             sm_scale = head_dim_og ** -0.5
         seq_dim = 1 if layout_flag == 0 else 2
         km = k.mean(dim=seq_dim, keepdim=True) if smooth_k else None
-        q_int8, q_scale, k_int8, k_scale = per_warp_int8_cuda(q, k, km, BLKQ=64, WARPQ=32, BLKK=64,
-                                                              tensor_layout=tensor_layout)
+        if qk_quant_gran == "per_thread":
+            # (core.py:204-205 of the reference pairs per-block scales, softmax scale folded in, with the kernel's
+            # per-thread path, whose shape check rejects them; here the scales are made at that granularity)
+            q_int8, q_scale, k_int8, k_scale = per_thread_int8(q, k, km, tensor_layout=tensor_layout)
+        else:
+            q_int8, q_scale, k_int8, k_scale = per_warp_int8_cuda(q, k, km, BLKQ=64, WARPQ=32, BLKK=64,
+                                                                  tensor_layout=tensor_layout)
         o = torch.empty(q.size(), dtype=dtype, device=q.device)
         lse = qattn.qk_int8_sv_f16_accum_f16_attn(q_int8, k_int8, v, o, q_scale, k_scale, layout_flag,
-                                                  1 if is_causal else 0, 2, sm_scale, 1 if return_lse else 0,
+                                                  1 if is_causal else 0, 3 if qk_quant_gran == "per_thread" else 2,
+                                                  sm_scale, 1 if return_lse else 0,
                                                   sparse, smooth_v=smooth_v, exact_exp=exact_exp,
                                                   two_waves=two_waves, pv_f16=pv_f16)
         o = o[..., :head_dim_og]

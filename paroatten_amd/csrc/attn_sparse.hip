@@ -60,9 +60,19 @@ template <int D> struct AttnLds {
 #define PARO_ATTN_WAVES_PER_SIMD ((D == 64 && !CAUSAL && !DUMP && !LSE) ? 3 : 2)
 
 // One 64-row q-block `vid` (numbered over batch, head, q-block) by one workgroup of two waves.
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
+//
+// PT: the scales have the reference's per-thread granularity (qk_quant_gran 3, csrc/qattn/
+// qk_int_sv_f16_cuda_sm80.cu:112-116 and :129-133): eight q scales per 32-row group, scale g for the rows
+// r with r % 8 == g (the rows lane / 4 + 8 j that a thread of the reference's m16n8 accumulator tiles holds),
+// and four k scales per 64-key block, scale j for the keys c with (c % 8) / 2 == j (the columns 2 (lane % 4),
+// 2 (lane % 4) + 1 of every 8-wide tile).  Here a lane holds one q-row, so its q scale is its own, and of its
+// 32 keys per block (offsets 4 lh + i % 4 within every group of 8) the even pair i % 4 < 2 has k scale 2 lh and
+// the odd pair 2 lh + 1.  Exact exponentials only.
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT, bool PT = false>
 __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) {
+  static_assert(!PT || (EXACT && !DUMP), "per-thread scales: exact exponentials, no score dump");
   using Lds = AttnLds<D>;
+  constexpr int CW = PT ? 4 : 1;    // k scales per key block
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
   constexpr int DT_TILES = D / 32;  // 32-channel tiles of O^T
   constexpr int NLD = D / 32;       // 16-byte pieces per thread per K (or V) tile
@@ -70,7 +80,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
 
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   float* clist = reinterpret_cast<float*>(smem + Lds::LIST_OFF);  // [nbk + LIST_PAD + 1] k_scale of kept blocks
-  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + p.nbk + Lds::LIST_PAD + 1);  // their indices
+  unsigned short* klist = reinterpret_cast<unsigned short*>(clist + (p.nbk + Lds::LIST_PAD + 1) * CW);  // their indices
 
   // (D = 64: opaque to the compiler.  In the paced kernel, which calls this in a loop, everything derived from
   // the lane number alone is otherwise computed once in front of that loop and kept in registers, 35 more than
@@ -93,18 +103,20 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   // loads whose only use sits in a branch are moved into it; so both waves build the (identical) lists, and
   // entries that are not kept go to a spare slot instead of being skipped.
   const int order_h = p.orders != nullptr ? p.orders[h] : 0;
-  const float* ksc_base = p.k_scale + bhk * p.nbk;
+  const float* ksc_base = p.k_scale + bhk * p.nbk * CW;
   const int kmax = CAUSAL ? min(p.nbk, qb + 1) : p.nbk;
   const uint8_t* mrow = p.sparse + b * p.sparse_bs + ((int64_t)h * p.nbq + qb) * p.nbk;
   constexpr int MU = 8;   // 64 x MU blocks per pass: one pass up to 512 blocks
   uint8_t m[MU];
   float msc[MU];
+  v4f msc4[PT ? MU : 1];
   auto list_load = [&](int base) {
 #pragma unroll
     for (int u = 0; u < MU; u++) {
       const int j = min(base + u * 64 + lane, kmax - 1);   // past the end: the last entry again
       m[u] = mrow[j];
-      msc[u] = ksc_base[j];
+      if constexpr (PT) msc4[u] = *reinterpret_cast<const v4f*>(ksc_base + 4 * j);
+      else msc[u] = ksc_base[j];
     }
   };
   const int trash = p.nbk + Lds::LIST_PAD;   // the spare slot
@@ -117,7 +129,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       const unsigned long long bal = __ballot(keep);
       const int pos = keep ? cnt + __popcll(bal & ((1ull << lane) - 1ull)) : trash;
       klist[pos] = (unsigned short)j;
-      clist[pos] = msc[u];
+      if constexpr (PT) *reinterpret_cast<v4f*>(clist + 4 * pos) = msc4[u];
+      else clist[pos] = msc[u];
       cnt += __popcll(bal);
     }
   };
@@ -132,7 +145,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const v4i*>(qp + 32 * ks);
   }
-  const float qsc = p.q_scale[((int64_t)b * p.H + h) * (p.nbq * 2) + qb * 2 + wave] * p.sm_scale_log2e;
+  const int64_t qs_group = ((int64_t)b * p.H + h) * (p.nbq * 2) + qb * 2 + wave;
+  const float qsc = (PT ? p.q_scale[qs_group * 8 + (l32 & 7)] : p.q_scale[qs_group]) * p.sm_scale_log2e;
 
   float* epi = reinterpret_cast<float*>(smem + Lds::EPI_OFF);   // [2][D]: v_scale, v_mean (D = 64)
   float epi_sc = 0.f, epi_mn = 0.f;
@@ -151,7 +165,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   // cnt - 1 of the lists just written; LDS operations of one wave complete in order)
   if (cnt > 0 && lane < Lds::LIST_PAD) {
     klist[cnt + lane] = klist[cnt - 1];
-    clist[cnt + lane] = clist[cnt - 1];
+    if constexpr (PT) *reinterpret_cast<v4f*>(clist + 4 * (cnt + lane)) = *reinterpret_cast<const v4f*>(clist + 4 * (cnt - 1));
+    else clist[cnt + lane] = clist[cnt - 1];
   }
   if constexpr (Lds::EPI_BYTES != 0) {
     epi[lane] = epi_sc;
@@ -314,7 +329,10 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     load_k(kb_2, 2);
     load_v(kb_1, 1);
   }
-  float c_cur = qsc * clist[0];
+  // (PT: the lane's two k scales of the block, for its even and its odd pairs of keys)
+  constexpr int CO = PT ? 1 : 0;
+  float c_cur = qsc * clist[PT ? 2 * lh : 0];
+  float cb_cur = qsc * clist[CO * (2 * lh + 1)];
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   read_k_frags(0);
@@ -357,12 +375,15 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       load_v(kb_2, svn);   // V(it+2) into the stage V(it-1) has left
     }
     const int kidx_v = (int)klist[it + 4];
-    const float c_next = qsc * clist[it + 1];
+    const float c_next = qsc * clist[(it + 1) * CW + (PT ? 2 * lh : 0)];
+    const float cb_next = qsc * clist[(it + 1) * CW + CO * (2 * lh + 1)];
     // scale of this block and what follows from it and from the current maximum alone
     const float c = c_cur;
+    const float cb = PT ? cb_cur : c;
     const float nmc = -S_MAGIC_F * c;
     const float c8 = (8.0f * FAST_FIELD_SCALE) * c;
     float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
+    float biasb = fmaf(-S_MAGIC_F, cb, m_off);
     float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: field = (8*(t + 7) + shift + 0.5) * 256 / 32767
 
     float s[2][16];
@@ -393,6 +414,18 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
 
     // Row maximum of the block (biased by 1.5*2^23 like the scores), as the log2-domain score m_blk
     auto block_max = [&]() {
+      if constexpr (PT) {
+        // the even and the odd pairs carry different scales: two maxima, scaled, then the larger one
+        float ma = fmaxf(s[0][0], s[0][1]), mb = fmaxf(s[0][2], s[0][3]);
+#pragma unroll
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+          for (int g = mt == 0 ? 1 : 0; g < 4; g++) {
+            ma = max3(ma, s[mt][4 * g], s[mt][4 * g + 1]);
+            mb = max3(mb, s[mt][4 * g + 2], s[mt][4 * g + 3]);
+          }
+        return partner_max(fmaxf(fmaf(ma, c, nmc), fmaf(mb, cb, -S_MAGIC_F * cb)));
+      }
       // four interleaved v_max3 chains (the values are integers read as floats: no NaN to canonicalise)
       float mx0 = max3(s[0][0], s[0][1], s[0][2]), mx1 = max3(s[0][8], s[0][9], s[0][10]);
       float mx2 = max3(s[1][0], s[1][1], s[1][2]), mx3 = max3(s[1][8], s[1][9], s[1][10]);
@@ -420,6 +453,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       m_off = P_EXP_OFFSET - m_new;
       m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT + 0.5f) * FAST_FIELD_SCALE;
       bias = fmaf(-S_MAGIC_F, c, m_off);
+      biasb = fmaf(-S_MAGIC_F, cb, m_off);
       bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
       if constexpr (LSE) d_exact *= alpha;
       d_acc[0] *= alpha;                                          // lanes 0..15: q-row lane
@@ -505,8 +539,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
         const int mt = r >> 2, i0 = 4 * (r & 3);
         const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
         const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
-        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], c, bias));
-        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], c, bias));
+        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], cb, biasb));
+        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], cb, biasb));
         if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
         int w;
         cvt_pk_fp8<false>(w, p0, p1);
@@ -557,6 +591,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     __builtin_amdgcn_s_barrier();
     kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3; kb_3 = kb_4;
     c_cur = c_next;
+    cb_cur = cb_next;
   };
 
   if constexpr (RING2) {
@@ -618,13 +653,13 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
   }
 }
 
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT, bool PT = false>
 __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_kernel(const AttnParams p) {
   // XCD-aware renumbering: hardware deals workgroup ids round-robin to the 8 XCDs
   const int per = gridDim.x >> 3;
   const int vid = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
   if (vid >= p.total) return;
-  attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>(p, vid);
+  attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT, PT>(p, vid);
 }
 
 // The same work with a resident set of workgroups per XCD that take the XCD's q-blocks generation by
@@ -723,10 +758,15 @@ static bool want_pacing(const AttnParams& p, int D) {
   return (int64_t)p.nbk * 64 * D * 2 > (int64_t)4 << 20;
 }
 
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
+// bytes of the kept-block list in LDS: per key block a 16-bit index and its k scale (four with per-thread scales)
+static size_t attn_list_bytes(int nbk, int list_pad, bool per_thread) {
+  return (((size_t)(nbk + list_pad + 1) * (per_thread ? 18 : 6) + 15) & ~(size_t)15);
+}
+
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT, bool PT = false>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
-  const size_t smem = AttnLds<D>::LIST_OFF + (((size_t)(p.nbk + AttnLds<D>::LIST_PAD + 1) * 6 + 15) & ~(size_t)15);
-  if (!DUMP && want_pacing(p, D)) {
+  const size_t smem = AttnLds<D>::LIST_OFF + attn_list_bytes(p.nbk, AttnLds<D>::LIST_PAD, PT);
+  if (!DUMP && !PT && want_pacing(p, D)) {
     auto kern = attn_sparse_paced_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
     if (smem > 48 * 1024)
       PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
@@ -755,12 +795,22 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
     }
   }
   const int grid = ((p.total + 7) / 8) * 8;
-  auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
+  auto kern = attn_sparse_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT, PT>;
   if (smem > 48 * 1024)
     PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(128), smem, st, p);
   PARO_HIP(hipGetLastError());
   return PARO_OK;
+}
+
+// per-thread scales (qk_quant_gran 3): the two-wave kernel with exact exponentials, plain launch
+template <int D, int OUT_DT>
+static int dispatch_attn_per_thread(const AttnParams& p, int is_causal, hipStream_t st) {
+  if (p.lse != nullptr)
+    return is_causal ? launch_attn<D, OUT_DT, true, false, true, true, true>(p, st)
+                     : launch_attn<D, OUT_DT, false, false, true, true, true>(p, st);
+  return is_causal ? launch_attn<D, OUT_DT, true, false, false, true, true>(p, st)
+                   : launch_attn<D, OUT_DT, false, false, false, true, true>(p, st);
 }
 
 template <int D, int OUT_DT>
@@ -791,10 +841,15 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
                             int64_t o_stride_n, float sm_scale, int is_causal, int flags, const int32_t* orders,
                             int n_text, int F, int Hh, int W, void* stream) {
   PARO_CHECK((flags & ~(PARO_ATTN_EXACT_EXP | PARO_ATTN_PACED | PARO_ATTN_UNPACED | PARO_ATTN_TWO_WAVES |
-                        PARO_ATTN_PV_F16)) == 0 &&
+                        PARO_ATTN_PV_F16 | PARO_ATTN_QK_PER_THREAD)) == 0 &&
                  (flags & (PARO_ATTN_PACED | PARO_ATTN_UNPACED)) != (PARO_ATTN_PACED | PARO_ATTN_UNPACED),
              PARO_ERR_INVALID_VALUE, "Unsupported attention flags: %d", flags);
   const bool pv16 = (flags & PARO_ATTN_PV_F16) != 0;
+  const bool per_thread = (flags & PARO_ATTN_QK_PER_THREAD) != 0;
+  PARO_CHECK(!per_thread || (!pv16 && s_dump == nullptr), PARO_ERR_UNSUPPORTED,
+             "per-thread scales (PARO_ATTN_QK_PER_THREAD) go with neither PARO_ATTN_PV_F16 nor the score dump");
+  PARO_CHECK(!per_thread || ((uintptr_t)k_scale % 16) == 0, PARO_ERR_RUNTIME,
+             "paro_attn_sparse_fwd: per-thread key scales must be 16-byte aligned");
   PARO_CHECK(q8 && k8 && v8 && q_scale && k_scale && (v_scale || pv16) && sparse && out, PARO_ERR_RUNTIME,
              "paro_attn_sparse_fwd: null tensor pointer");
   PARO_CHECK(!pv16 || s_dump == nullptr, PARO_ERR_UNSUPPORTED, "the score dump is not available with PARO_ATTN_PV_F16");
@@ -821,10 +876,10 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
                  (int64_t)nbk * 64 * D < (int64_t)1 << 31,
              PARO_ERR_RUNTIME, "paro_attn_sparse_fwd: one head of key/value spans 2 GiB or more (kv_len %d, stride %lld)",
              Nk, (long long)k_stride_n);
-  // ring stages + the list of kept blocks (6 bytes each) have to fit the 160 KB of LDS of one CU
+  // ring stages + the list of kept blocks (6 bytes each, 18 with per-thread scales) have to fit the 160 KB of LDS of one CU
   if (!pv16) {
     const int64_t ring = D == 128 ? 2 * 2 * 64 * 128 : 3 * 2 * 64 * 64;
-    PARO_CHECK(ring + ((int64_t)nbk + 8) * 6 + 64 <= 160 * 1024, PARO_ERR_RUNTIME,
+    PARO_CHECK(ring + (per_thread ? ((int64_t)nbk + 9) * 18 + 1024 : ((int64_t)nbk + 8) * 6 + 64) <= 160 * 1024, PARO_ERR_RUNTIME,
                "kv_len %d: the list of %d key blocks does not fit the local data share", Nk, nbk);
   }
   AttnParams p;
@@ -843,6 +898,13 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
   const bool exact = (flags & PARO_ATTN_EXACT_EXP) != 0;
   // float16 P.V product: a kernel of its own (true exponentials, plain launch)
   if (pv16) return launch_attn_pv16(p, D, out_dtype, is_causal != 0, st);
+  if (per_thread) {
+    if (D == 64)
+      return out_dtype == PARO_DTYPE_F16 ? dispatch_attn_per_thread<64, PARO_DTYPE_F16>(p, is_causal, st)
+                                         : dispatch_attn_per_thread<64, PARO_DTYPE_BF16>(p, is_causal, st);
+    return out_dtype == PARO_DTYPE_F16 ? dispatch_attn_per_thread<128, PARO_DTYPE_F16>(p, is_causal, st)
+                                       : dispatch_attn_per_thread<128, PARO_DTYPE_BF16>(p, is_causal, st);
+  }
   // D = 64 without lse or score dump: one wave per q-block (attn_sparse_w64.hip), unless the caller asks for the
   // two-wave kernel or the launch is to be paced (only the two-wave kernel has the paced form)
   if (D == 64 && lse == nullptr && !dump && (flags & PARO_ATTN_TWO_WAVES) == 0 && !want_pacing(p, D))
@@ -915,8 +977,7 @@ extern "C" int paro_qk_int8_sv_f16_attn(const int8_t* q8, const int8_t* k8, cons
   PARO_CHECK(tensor_layout == 0 || tensor_layout == 1, PARO_ERR_INVALID_VALUE, "tensor_layout must be 0 or 1");
   PARO_CHECK(qk_quant_gran == 2 || qk_quant_gran == 3, PARO_ERR_INVALID_VALUE, "Unsupported quantization granularity: %d",
              qk_quant_gran);
-  PARO_CHECK(qk_quant_gran == 2, PARO_ERR_UNSUPPORTED,
-             "qk_quant_gran=3 (per_thread) is not implemented: quantise with per_warp (gran 2)");
+  if (qk_quant_gran == 3) flags |= PARO_ATTN_QK_PER_THREAD;
   PARO_CHECK(workspace && ((uintptr_t)workspace % 256) == 0, PARO_ERR_RUNTIME,
              "paro_qk_int8_sv_f16_attn: workspace must be a 256-byte aligned device buffer");
   PARO_CHECK(B > 0 && Hkv > 0 && Nk > 0 && (D == 64 || D == 128), PARO_ERR_INVALID_VALUE,

@@ -112,6 +112,11 @@ torch::Tensor qk_int8_sv_f16_accum_f16_attn(torch::Tensor query, torch::Tensor k
     shape(query_scale, "query_scale", {B, H, nbq * 2},
           "batch_size, num_qo_heads, div_ceil(qo_len, CTA_Q) * (CTA_Q / WARP_Q)");
     shape(key_scale, "key_scale", {B, Hkv, nbk}, "batch_size, num_kv_heads, div_ceil(kv_len, CTA_K) * (CTA_K / WARP_K)");
+  } else if (qk_quant_gran == 3) {   // per thread (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:1034-1038)
+    shape(query_scale, "query_scale", {B, H, nbq * 2 * 8},
+          "batch_size, num_qo_heads, div_ceil(qo_len, CTA_Q) * (CTA_Q / WARP_Q) * 8");
+    shape(key_scale, "key_scale", {B, Hkv, nbk * 4},
+          "batch_size, num_kv_heads, div_ceil(kv_len, CTA_K) * (CTA_K / WARP_K) * 4");
   }
   // the reference reads `sparse` through a raw pointer without any check
   on_gpu(sparse, "sparse"); contiguous(sparse, "sparse");

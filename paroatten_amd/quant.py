@@ -67,6 +67,42 @@ def per_warp_int8(q, k, km: Optional[torch.Tensor] = None, BLKQ: int = 128, WARP
     return q_int8, q_scale, k_int8, k_scale
 
 
+def per_thread_int8(q, k, km: Optional[torch.Tensor] = None, tensor_layout: str = "HND"):
+    """Scales of the attention kernel's per-thread granularity (qk_quant_gran 3: csrc/qattn/
+    qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133, shapes :1034-1038): eight per 32 query tokens (scale g for the
+    tokens r with r % 8 == g), four per 64 key tokens (scale j for the tokens c with (c % 8) / 2 == j), the same
+    arithmetic as per_warp_int8 otherwise.  The reference has no quantiser of this granularity (its
+    paroattention/core.py:204-205 calls the per-block one); the grouping is the one its kernel's indexing implies.
+    Returns (q_int8, q_scale [B,Hq,ceil(Nq/64)*16], k_int8, k_scale [B,Hkv,ceil(Nk/64)*4])."""
+    layout_flag = 0 if tensor_layout == "NHD" else 1
+    outs = []
+    for x, mean, is_key in ((q, None, 0), (k, km, 1)):
+        b, h, n, d = _dims(x, tensor_layout)
+        _lib.require_gpu(x, "k" if is_key else "q")
+        if x.dtype not in (torch.float16, torch.bfloat16):
+            raise RuntimeError(f"per_thread_int8 failed to dispatch data type {x.dtype}")
+        if d not in (64, 128):
+            raise ValueError(f"Unsupported head dim: {d}")
+        if x.stride(-1) != 1:
+            raise RuntimeError("Tensor input must be contiguous at the last dimension")
+        x8 = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+        scale = torch.empty((b, h, (n + 63) // 64 * (4 if is_key else 16)), dtype=torch.float32, device=x.device)
+        xs_n, xs_h = (x.stride(1), x.stride(2)) if layout_flag == 0 else (x.stride(2), x.stride(1))
+        os_n, os_h = (x8.stride(1), x8.stride(2)) if layout_flag == 0 else (x8.stride(2), x8.stride(1))
+        ms_b = ms_h = 0
+        if mean is not None:
+            mean = mean.squeeze(1) if layout_flag == 0 else mean.squeeze(2)
+            if tuple(mean.shape) != (b, h, d) or mean.dtype != x.dtype or mean.stride(-1) != 1:
+                raise RuntimeError("Tensor mean must have shape (batch_size, num_heads, head_dim), the input's dtype "
+                                   "and a contiguous last dimension")
+            ms_b, ms_h = mean.stride(0), mean.stride(1)
+        _lib.on(x).paro_quant_int8_per_thread(ptr(x), _lib.DTYPE_CODE[x.dtype], ptr(mean), ptr(x8), ptr(scale), b, h, n, d,
+                                              x.stride(0), xs_h, xs_n, ms_b, ms_h, x8.stride(0), os_h, os_n, is_key,
+                                              stream_of(x))
+        outs += [x8, scale]
+    return tuple(outs)
+
+
 def sub_mean(v: torch.Tensor, tensor_layout: str = "HND"):
     """(v - mean over tokens) as float16, and the mean in v's dtype (paroattention/quant.py:182-222)."""
     layout_flag = 0 if tensor_layout == "NHD" else 1

@@ -90,11 +90,16 @@ def test_c_abi_argument_errors_without_gpu():
     assert rc == L.PARO_ERR_INVALID_VALUE and b"scale_max" in lib.paro_last_error()
     rc = lib.paro_permute_inv(p, p, 0, p, 1, 1, 100, 64, 10, 3, 5, 7, 0, 0, 64, 0, 0, 64, None)
     assert rc == L.PARO_ERR_RUNTIME and b"does not equal the token count" in lib.paro_last_error()
-    rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
-                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 3, 0.125, 1, 0, None)
-    assert rc == L.PARO_ERR_UNSUPPORTED
+    # per-thread scales go with neither the float16 P.V product nor the score dump
+    rc = lib.paro_attn_sparse_fwd(p, p, p, p, p, p, p, p, 0, p, 0, None, None, 1, 1, 1, 64, 64, 64,
+                                  0, 0, 64, 0, 0, 64, 0, 0, 64, 0.125, 0,
+                                  L.PARO_ATTN_PV_F16 | L.PARO_ATTN_QK_PER_THREAD, None)
+    assert rc == L.PARO_ERR_UNSUPPORTED and b"per-thread" in lib.paro_last_error()
     with pytest.raises(NotImplementedError):
         L.check(rc)
+    rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 1 << 30, 1, 1, 1, 64, 64, 64,
+                                      0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 4, 0.125, 1, 0, None)
+    assert rc == L.PARO_ERR_INVALID_VALUE and b"granularity" in lib.paro_last_error()
     rc = lib.paro_qk_int8_sv_f16_attn(p, p, p, 0, p, 0, p, p, p, 0, None, p, 16, 1, 1, 1, 64, 64, 64,
                                       0, 0, 64, 0, 0, 64, 0, 0, 64, 0, 0, 64, 1, 0, 2, 0.125, 1, 0, None)
     assert rc == L.PARO_ERR_RUNTIME and b"workspace" in lib.paro_last_error()

@@ -106,8 +106,16 @@ def test_extension_matches_ctypes_mirrors_bit_for_bit(ext, dev):
         ext._qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, torch.empty_like(q), qs, ks, 7, 0, 2, 0.125, 0, mask)
     with pytest.raises(RuntimeError, match="Tensor sparse must have shape"):
         ext._qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, torch.empty_like(q), qs, ks, 1, 0, 2, 0.125, 0, mask[:, :3].contiguous())
-    with pytest.raises(NotImplementedError):
+    # per-thread granularity: the reference's shape check (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:1034-1038), then the
+    # same result as the ctypes mirror
+    with pytest.raises(RuntimeError, match=r"Tensor query_scale must have shape .*\* 8"):
         ext._qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, torch.empty_like(q), qs, ks, 1, 0, 3, 0.125, 0, mask)
+    from paroatten_amd import quant
+    q8t, qst, k8t, kst = quant.per_thread_int8(q, k, km.unsqueeze(2))
+    a, b = torch.empty_like(q), torch.empty_like(q)
+    la = ext._qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8t, k8t, v, a, qst, kst, 1, 0, 3, D ** -0.5, 1, mask)
+    lb = _qattn_sm80.qk_int8_sv_f16_accum_f16_attn(q8t, k8t, v, b, qst, kst, 1, 0, 3, D ** -0.5, 1, mask)
+    assert torch.equal(a, b) and torch.equal(la, lb)
 
     # _rope.rope_permutation on the side stream torch is currently on
     g = torch.Generator(device=dev).manual_seed(5)

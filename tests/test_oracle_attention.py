@@ -131,3 +131,40 @@ def test_paro_path_equals_unpermuted_attention_when_mask_is_dense():
     o = O.paro_path(q, k, v, mask, plan, 0, grid, n_text)
     full = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
     assert torch.nn.functional.cosine_similarity(o.float().flatten(), full.flatten(), dim=0) > 0.995
+
+
+def test_per_thread_scales_reduce_to_per_warp_and_to_rowwise_dequantisation():
+    """sparse_attention(per_thread=True): (i) with scales that are constant over each 32-row / 64-key group it
+    is the per-warp result bit for bit; (ii) with distinct scales it is fp64 softmax attention on Q and K
+    dequantised row by row with the scale the reference kernel's lanes read for that row (enumerated lane by
+    lane in test_oracle_quant, not taken from the oracle's index law)."""
+    from test_oracle_quant import _lane_enumeration
+    g = torch.Generator().manual_seed(11)
+    B, H, Hk, N, D = 1, 4, 2, 200, 64
+    q = torch.randn(B, H, N, D, generator=g).to(torch.float16)
+    k = torch.randn(B, Hk, N, D, generator=g).to(torch.float16)
+    v = torch.randn(B, Hk, N, D, generator=g).to(torch.float16)
+    nb = (N + 63) // 64
+    mask = synth.make_block_mask(H, nb, 0.6, seed=3)[None].contiguous()
+    q8, qs, k8, ks = O.per_warp_int8(q, k, BLKQ=64, WARPQ=32, BLKK=64)
+    o2, l2 = O.sparse_attention(q8, k8, v, qs, ks, mask, D ** -0.5)
+    o3, l3 = O.sparse_attention(q8, k8, v, qs.repeat_interleave(8, dim=2), ks.repeat_interleave(4, dim=2), mask,
+                                D ** -0.5, per_thread=True)
+    assert torch.equal(o2, o3) and torch.equal(l2, l3)
+
+    q8, qs, k8, ks = O.per_thread_int8(q, k)
+    assert qs.shape == (B, H, nb * 16) and ks.shape == (B, Hk, nb * 4)
+    assert len(torch.unique(qs[0, 0, :8])) == 8 and len(torch.unique(ks[0, 0, :4])) == 4   # distinct scales
+    o, lse = O.sparse_attention(q8, k8, v, qs, ks, mask, D ** -0.5, per_thread=True, compute_dtype=torch.float64)
+    qi, ki = _lane_enumeration(N, False), _lane_enumeration(N, True)
+    qd = q8.double() * qs.double()[:, :, qi].unsqueeze(-1)
+    kd = (k8.double() * ks.double()[:, :, ki].unsqueeze(-1)).repeat_interleave(H // Hk, dim=1)
+    s = qd @ kd.transpose(-1, -2) * D ** -0.5
+    keep = O.expand_block_mask(mask, N, N)
+    s = s.masked_fill(~keep, float("-inf"))
+    want = torch.softmax(s, dim=-1) @ v.double().repeat_interleave(H // Hk, dim=1)
+    assert torch.allclose(o.double(), want, atol=2e-3, rtol=0)   # fp16 rounding of the output
+    assert torch.allclose(lse.double(), torch.logsumexp(s, dim=-1) * O.LOG2E, atol=1e-4, rtol=1e-6)
+    # and it is not what per-warp indexing of the same scale tensors would give
+    o_wrong, _ = O.sparse_attention(q8, k8, v, qs[:, :, ::8].contiguous(), ks[:, :, ::4].contiguous(), mask, D ** -0.5)
+    assert (o_wrong.float() - o.float()).abs().max() > 1e-2

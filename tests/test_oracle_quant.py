@@ -104,3 +104,70 @@ def test_ties_round_to_even():
     q8, sc = O.quant_int8(x, 16)
     assert q8[0, 0, 0, :8].tolist() == [127, 0, 2, 2, 0, -2, -2, 4]
     assert float(sc) == 1.0
+
+
+def _lane_enumeration(n, is_key):
+    """Scale index per token from an enumeration of the reference kernel's accumulator lanes, the way its
+    per-thread branch reads them (csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116: q_scale_idx = ... +
+    warp_idx_q * 8 + lane_id / 4, :129-133: k_scale_idx = ... + lane_id % 4, advancing by 4 per 64-key block):
+    lane l of a warp holds, in every m16n8 tile, rows l/4 and l/4 + 8 and columns 2*(l%4), 2*(l%4) + 1."""
+    idx = [-1] * n
+    if is_key:
+        for block in range((n + 63) // 64):
+            for lane in range(32):
+                for tile in range(8):              # 8-column tiles of the 64-key block
+                    for e in range(2):
+                        c = block * 64 + tile * 8 + 2 * (lane % 4) + e
+                        if c < n:
+                            idx[c] = block * 4 + lane % 4
+    else:
+        for warp in range((n + 31) // 32):
+            for lane in range(32):
+                for tile in range(2):              # 16-row tiles of the 32-row warp
+                    for half in range(2):
+                        r = warp * 32 + tile * 16 + lane // 4 + 8 * half
+                        if r < n:
+                            idx[r] = warp * 8 + lane // 4
+    assert min(idx) >= 0
+    return torch.tensor(idx)
+
+
+@pytest.mark.parametrize("n", [1, 31, 64, 100, 257])
+def test_per_thread_scale_index_matches_the_lane_enumeration(n):
+    assert torch.equal(O.per_thread_scale_index(n, False), _lane_enumeration(n, False))
+    assert torch.equal(O.per_thread_scale_index(n, True), _lane_enumeration(n, True))
+    # the values a wrong law would give differ: plain 8-row groups, or pairs of 16 consecutive keys
+    if n >= 64:
+        assert not torch.equal(O.per_thread_scale_index(n, False), torch.arange(n) // 4)
+        assert not torch.equal(O.per_thread_scale_index(n, True), torch.arange(n) // 16)
+
+
+@pytest.mark.parametrize("is_key", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_per_thread_quantiser_is_quant_int8_on_regrouped_tokens(is_key, dtype):
+    """Tokens sorted so that every per-thread group is contiguous turn the per-thread quantiser into the
+    pinned group quantiser (groups of 4 query tokens / 16 key tokens); a ragged length equals its zero-padded
+    self on the tokens that exist."""
+    g = torch.Generator().manual_seed(5)
+    B, H, N, D = 2, 3, 192, 64
+    x = (torch.randn(B, H, N, D, generator=g) * torch.rand(1, 1, N, 1, generator=g) * 3).to(dtype)
+    mean = x.float().mean(dim=2).to(dtype) if is_key else None
+    q8, sc = O.quant_int8_per_thread(x, is_key, mean=mean)
+    idx = _lane_enumeration(N, is_key)
+    order = torch.argsort(idx, stable=True)                   # tokens of scale 0, then of scale 1, ...
+    per = 16 if is_key else 4
+    assert torch.equal(idx[order], torch.arange(N // per).repeat_interleave(per))
+    q8_ref, sc_ref = O.quant_int8(x[:, :, order], per, mean=mean)
+    assert torch.equal(sc, sc_ref)
+    assert torch.equal(q8[:, :, order], q8_ref)
+    assert sc.shape == (B, H, N // 64 * (4 if is_key else 16))
+    # ragged
+    n = 150
+    q8r, scr = O.quant_int8_per_thread(x[:, :, :n], is_key, mean=mean)
+    xz = x.clone()
+    if mean is not None:
+        xz[:, :, n:] = mean[:, :, None, :]                    # x - mean = 0 exactly there
+    else:
+        xz[:, :, n:] = 0
+    q8z, scz = O.quant_int8_per_thread(xz, is_key, mean=mean)
+    assert torch.equal(q8r, q8z[:, :, :n]) and torch.equal(scr, scz)
