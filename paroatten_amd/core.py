@@ -42,7 +42,7 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
     [B,Hq,ceil(Nq/64),ceil(Nk/64)] or [Hq,..] shared by the batch, True = compute that 64x64 block.
     Returns o (q's dtype and shape) or (o, lse) with lse the natural-log sum-exp per row.
     smooth_k subtracts the per-(batch,head) token mean of K before quantisation (softmax is
-    invariant to it); smooth_v does the same for V inside the FP8 conversion and adds the mean back;
+    invariant to it; the returned lse is corrected by sm_scale * q . mean, so it is that of the given q and k); smooth_v does the same for V inside the FP8 conversion and adds the mean back;
     exact_exp trades speed for fp32-evaluated softmax exponentials (see _qattn_sm80); two_waves picks the
     two-waves-per-q-block kernel where the library would take the one-wave one (bit-identical results);
     pv_f16 is the accuracy mode: the P.V product in float16 with fp32 accumulation, as the reference computes
@@ -94,5 +94,19 @@ def paroattn_qk_int8_pv_fp16_cuda(q, k, v, sparse, tensor_layout: str = "HND", i
                                                   two_waves=two_waves, pv_f16=pv_f16)
         o = o[..., :head_dim_og]
         if return_lse:
-            return o, lse / 1.44269504
+            lse = lse / 1.44269504
+            if km is not None:
+                # the kernel saw K - km: every score of row i is lower by sm_scale * q_i . km, which the softmax
+                # does not notice but the log-sum-exp does; put it back, so that lse is that of the scores of q
+                # and k as given (what a caller that merges partial results over key ranges needs)
+                groups = q.size(2 if layout_flag == 0 else 1) // km.size(2 if layout_flag == 0 else 1)
+                if layout_flag == 0:   # q [B,N,H,D], km [B,1,Hkv,D]
+                    kmh = km.float().repeat_interleave(groups, dim=2)
+                    corr = torch.stack([(q[b].float() * kmh[b]).sum(-1).transpose(0, 1) for b in range(q.size(0))])
+                else:                  # q [B,H,N,D], km [B,Hkv,1,D]
+                    kmh = km.float().repeat_interleave(groups, dim=1)
+                    corr = torch.stack([torch.bmm(q[b].float(), kmh[b].transpose(1, 2)).squeeze(-1)
+                                        for b in range(q.size(0))])
+                lse = lse + corr * sm_scale
+            return o, lse
         return o

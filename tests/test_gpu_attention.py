@@ -34,7 +34,13 @@ def _run(dev, B, H, N, D, dtype, density, seed, Hkv=None, causal=False, smooth_k
     out = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), m_dev, is_causal=causal,
                                           smooth_k=smooth_k, return_lse=return_lse, exact_exp=exact_exp)
     o, lse = out if return_lse else (out, None)
-    return o.cpu(), (None if lse is None else lse.cpu()), (o_ref, a_ref), lse_ref / O.LOG2E, mask_b
+    lse_ref = lse_ref / O.LOG2E
+    if smooth_k:
+        # the operator returns the log-sum-exp of the scores of q and k as given: the oracle's, taken on K - km,
+        # plus sm_scale * q . km per row
+        lse_ref = lse_ref + torch.einsum("bhnd,bhd->bhn", q.float(),
+                                         km.float().squeeze(2).repeat_interleave(H // Hkv, dim=1)) * D ** -0.5
+    return o.cpu(), (None if lse is None else lse.cpu()), (o_ref, a_ref), lse_ref, mask_b
 
 
 def _assert_close(o, ref, baseline_shape=False):
@@ -101,6 +107,34 @@ def test_empty_rows_and_single_block(dev):
     keep = ~torch.isinf(lse_ref)
     assert torch.equal(torch.isinf(lse), torch.isinf(lse_ref))
     assert torch.allclose(lse[keep], lse_ref[keep], atol=2e-3, rtol=1e-4)
+
+
+def test_lse_with_k_smoothing_is_that_of_the_unsmoothed_scores(dev):
+    """K smoothing lowers every score of row i by sm_scale * q_i . km: invisible to the softmax, not to the
+    log-sum-exp.  The operator puts it back: its lse with smooth_k=True agrees with the lse of the same call without
+    smoothing up to the INT8 rounding of the two different K tensors, and with the oracle's lse of unsmoothed
+    quantised scores; left out, the difference would be of order 1 (the K of the synthetic inputs carries a bias)."""
+    import paroatten_amd as P
+    B, H, Hkv, N, D = 1, 4, 2, 900, 64
+    q, _, _ = synth.make_qkv(B, H, N, D, torch.float16, seed=21)
+    _, k, v = synth.make_qkv(B, Hkv, N, D, torch.float16, seed=22)
+    nb = (N + 63) // 64
+    mask = synth.make_block_mask(H, nb, 0.5, seed=23)
+    qd, kd, vd, md = q.to(dev), k.to(dev), v.to(dev), mask.to(dev)
+    lse_s = P.paroattn_qk_int8_pv_fp16_cuda(qd, kd, vd, md, smooth_k=True, return_lse=True)[1].cpu()
+    lse_u = P.paroattn_qk_int8_pv_fp16_cuda(qd, kd, vd, md, smooth_k=False, return_lse=True)[1].cpu()
+    tr = lambda t: t.transpose(1, 2).contiguous()
+    lse_n = P.paroattn_qk_int8_pv_fp16_cuda(tr(qd), tr(kd), tr(vd), md, tensor_layout="NHD", smooth_k=True,
+                                            return_lse=True)[1].cpu()
+    q8, qs, k8, ks = O.per_warp_int8(q, k, km=None, BLKQ=64, WARPQ=32, BLKK=64)
+    _, lse_o = O.sparse_attention(q8, k8, v, qs, ks, mask[None], D ** -0.5)
+    # (the unsmoothed K spends most of its INT8 range on the bias: its scores carry a rounding noise of a few 1e-2)
+    for other in (lse_u, lse_o / O.LOG2E):
+        d = (lse_s - other).abs()
+        assert float(d.max()) < 0.2 and float(d.mean()) < 0.03, (float(d.max()), float(d.mean()))
+    assert torch.allclose(lse_n, lse_s, atol=1e-4, rtol=1e-5)      # the correction is summed in another order
+    corr = torch.einsum("bhnd,bhd->bhn", q.float(), k.float().mean(dim=2).repeat_interleave(H // Hkv, dim=1)) * D ** -0.5
+    assert float(corr.abs().mean()) > 0.3      # what an uncorrected lse would be off by
 
 
 def test_causal_and_gqa(dev):

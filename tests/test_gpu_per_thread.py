@@ -69,7 +69,8 @@ def test_per_thread_attention_against_oracle(dev, B, H, Hkv, N, D, dtype, densit
     o, lse = out if lse_on else (out, None)
     assert_attention_close(o.cpu(), o_ref, a_ref, 0.999, what="per_thread")
     if lse_on:
-        lr = lse_ref / O.LOG2E
+        lr = lse_ref / O.LOG2E + torch.einsum("bhnd,bhd->bhn", q.float(),
+                                              km.float().squeeze(2).repeat_interleave(H // Hkv, dim=1)) * D ** -0.5
         assert torch.equal(torch.isinf(lse.cpu()), torch.isinf(lr))
         keep = ~torch.isinf(lr)
         assert torch.allclose(lse.cpu()[keep], lr[keep], atol=2e-3, rtol=1e-4)
