@@ -67,10 +67,10 @@ template <int D> struct AttnLds {
 // and four k scales per 64-key block, scale j for the keys c with (c % 8) / 2 == j (the columns 2 (lane % 4),
 // 2 (lane % 4) + 1 of every 8-wide tile).  Here a lane holds one q-row, so its q scale is its own, and of its
 // 32 keys per block (offsets 4 lh + i % 4 within every group of 8) the even pair i % 4 < 2 has k scale 2 lh and
-// the odd pair 2 lh + 1.  Exact exponentials only.
+// the odd pair 2 lh + 1: two affine maps from score to exponent per block instead of one.
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT, bool PT = false>
 __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) {
-  static_assert(!PT || (EXACT && !DUMP), "per-thread scales: exact exponentials, no score dump");
+  static_assert(!PT || !DUMP, "per-thread scales: no score dump");
   using Lds = AttnLds<D>;
   constexpr int CW = PT ? 4 : 1;    // k scales per key block
   constexpr int KS = D / 32;        // k-steps of the QK MFMA (32 channels each)
@@ -385,6 +385,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
     float biasb = fmaf(-S_MAGIC_F, cb, m_off);
     float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: field = (8*(t + 7) + shift + 0.5) * 256 / 32767
+    const float c8b = PT ? (8.0f * FAST_FIELD_SCALE) * cb : c8;
+    float bias8b = fmaf(-S_MAGIC_F, c8b, m_off8);
 
     float s[2][16];
 #pragma unroll
@@ -455,6 +457,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       bias = fmaf(-S_MAGIC_F, c, m_off);
       biasb = fmaf(-S_MAGIC_F, cb, m_off);
       bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
+      bias8b = fmaf(-S_MAGIC_F, c8b, m_off8);
       if constexpr (LSE) d_exact *= alpha;
       d_acc[0] *= alpha;                                          // lanes 0..15: q-row lane
       d_acc[1] *= __shfl(alpha, (lane & 15) + 16, 64);            // and q-row lane+16
@@ -487,7 +490,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       auto fast_words = [&]() {
         float u_cur[4], u_nxt[4];
 #pragma unroll
-        for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], c8, bias8);
+        for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], q < 2 ? c8 : c8b, q < 2 ? bias8 : bias8b);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
@@ -496,13 +499,13 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
           const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
           if (rn < 8) {
             u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
-            u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8, bias8);
+            u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8b, bias8b);
           }
           const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
           __builtin_amdgcn_sched_barrier(0);
           if (rn < 8) {
             u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
-            u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8, bias8);
+            u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8b, bias8b);
           }
           const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
           __builtin_amdgcn_sched_barrier(0);
@@ -803,14 +806,17 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
   return PARO_OK;
 }
 
-// per-thread scales (qk_quant_gran 3): the two-wave kernel with exact exponentials, plain launch
+// per-thread scales (qk_quant_gran 3): the two-wave kernel, plain launch
 template <int D, int OUT_DT>
-static int dispatch_attn_per_thread(const AttnParams& p, int is_causal, hipStream_t st) {
+static int dispatch_attn_per_thread(const AttnParams& p, int is_causal, bool exact, hipStream_t st) {
   if (p.lse != nullptr)
     return is_causal ? launch_attn<D, OUT_DT, true, false, true, true, true>(p, st)
                      : launch_attn<D, OUT_DT, false, false, true, true, true>(p, st);
-  return is_causal ? launch_attn<D, OUT_DT, true, false, false, true, true>(p, st)
-                   : launch_attn<D, OUT_DT, false, false, false, true, true>(p, st);
+  if (exact)
+    return is_causal ? launch_attn<D, OUT_DT, true, false, false, true, true>(p, st)
+                     : launch_attn<D, OUT_DT, false, false, false, true, true>(p, st);
+  return is_causal ? launch_attn<D, OUT_DT, true, false, false, false, true>(p, st)
+                   : launch_attn<D, OUT_DT, false, false, false, false, true>(p, st);
 }
 
 template <int D, int OUT_DT>
@@ -900,10 +906,10 @@ static int attn_sparse_impl(const int8_t* q8, const int8_t* k8, const uint8_t* v
   if (pv16) return launch_attn_pv16(p, D, out_dtype, is_causal != 0, st);
   if (per_thread) {
     if (D == 64)
-      return out_dtype == PARO_DTYPE_F16 ? dispatch_attn_per_thread<64, PARO_DTYPE_F16>(p, is_causal, st)
-                                         : dispatch_attn_per_thread<64, PARO_DTYPE_BF16>(p, is_causal, st);
-    return out_dtype == PARO_DTYPE_F16 ? dispatch_attn_per_thread<128, PARO_DTYPE_F16>(p, is_causal, st)
-                                       : dispatch_attn_per_thread<128, PARO_DTYPE_BF16>(p, is_causal, st);
+      return out_dtype == PARO_DTYPE_F16 ? dispatch_attn_per_thread<64, PARO_DTYPE_F16>(p, is_causal, exact, st)
+                                         : dispatch_attn_per_thread<64, PARO_DTYPE_BF16>(p, is_causal, exact, st);
+    return out_dtype == PARO_DTYPE_F16 ? dispatch_attn_per_thread<128, PARO_DTYPE_F16>(p, is_causal, exact, st)
+                                       : dispatch_attn_per_thread<128, PARO_DTYPE_BF16>(p, is_causal, exact, st);
   }
   // D = 64 without lse or score dump: one wave per q-block (attn_sparse_w64.hip), unless the caller asks for the
   // two-wave kernel or the launch is to be paced (only the two-wave kernel has the paced form)

@@ -57,7 +57,12 @@ def _oracle(q, k, v, mask, D, causal, smooth_k):
     mask_b = mask[None].expand(B, *mask.shape).contiguous()
     # the kernel multiplies by V in float16: for bfloat16 inputs that conversion is exact at these magnitudes
     o_ref, lse_ref = O.sparse_attention(q8, k8, v, qs, ks, mask_b, D ** -0.5, is_causal=causal, out_dtype=torch.float32)
-    return o_ref, lse_ref / O.LOG2E
+    lse_ref = lse_ref / O.LOG2E
+    if smooth_k:   # the operator returns the log-sum-exp of the scores of q and k as given (K - km + km)
+        H, Hkv = q.size(1), k.size(1)
+        lse_ref = lse_ref + torch.einsum("bhnd,bhd->bhn", q.float(),
+                                         km.float().squeeze(2).repeat_interleave(H // Hkv, dim=1)) * D ** -0.5
+    return o_ref, lse_ref
 
 
 @pytest.mark.parametrize("D,dtype,N,Hkv,causal", [

@@ -44,14 +44,16 @@ def test_per_thread_quantiser_bitexact(dev, D, N, dtype, layout, smooth):
         assert float(want[1][0, 0, :8].max() / want[1][0, 0, :8].min()) > 1.05
 
 
-@pytest.mark.parametrize("B,H,Hkv,N,D,dtype,density,causal,lse_on", [
-    (2, 3, 3, 1000, 64, torch.float16, 0.4, False, True),
-    (1, 4, 2, 700, 64, torch.bfloat16, 1.0, True, False),
-    (1, 2, 2, 2048, 128, torch.bfloat16, 0.3, False, False),
-    (2, 2, 1, 333, 128, torch.float16, 0.6, True, True),
-    (1, 2, 2, 63, 64, torch.float16, 1.0, False, True),
+@pytest.mark.parametrize("B,H,Hkv,N,D,dtype,density,causal,lse_on,exact", [
+    (2, 3, 3, 1000, 64, torch.float16, 0.4, False, True, False),     # (lse: true exponentials)
+    (1, 4, 2, 700, 64, torch.bfloat16, 1.0, True, False, False),     # fast construction of the weights
+    (1, 2, 2, 2048, 128, torch.bfloat16, 0.3, False, False, False),
+    (1, 2, 2, 2048, 128, torch.bfloat16, 0.3, False, False, True),   # true exponentials without lse
+    (2, 2, 1, 333, 128, torch.float16, 0.6, True, True, False),
+    (1, 2, 2, 63, 64, torch.float16, 1.0, False, True, False),
+    (1, 3, 3, 1500, 64, torch.float16, 0.3, False, False, True),
 ])
-def test_per_thread_attention_against_oracle(dev, B, H, Hkv, N, D, dtype, density, causal, lse_on):
+def test_per_thread_attention_against_oracle(dev, B, H, Hkv, N, D, dtype, density, causal, lse_on, exact):
     import paroatten_amd as P
     q, k, v = _inputs(B, H, Hkv, N, D, dtype, seed=N)
     nb = (N + 63) // 64
@@ -65,7 +67,7 @@ def test_per_thread_attention_against_oracle(dev, B, H, Hkv, N, D, dtype, densit
     a_ref, _ = O.sparse_attention(q8, k8, v.abs(), qs, ks, mask_b, D ** -0.5, is_causal=causal, out_dtype=torch.float32,
                                   per_thread=True)
     out = P.paroattn_qk_int8_pv_fp16_cuda(q.to(dev), k.to(dev), v.to(dev), mask.to(dev), is_causal=causal,
-                                          qk_quant_gran="per_thread", smooth_k=True, return_lse=lse_on)
+                                          qk_quant_gran="per_thread", smooth_k=True, return_lse=lse_on, exact_exp=exact)
     o, lse = out if lse_on else (out, None)
     assert_attention_close(o.cpu(), o_ref, a_ref, 0.999, what="per_thread")
     if lse_on:
@@ -95,6 +97,11 @@ def test_per_thread_with_group_constant_scales_is_the_per_warp_kernel(dev):
     lb = qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, b, qs.repeat_interleave(8, dim=2).contiguous(),
                                              ks.repeat_interleave(4, dim=2).contiguous(), 1, 0, 3, D ** -0.5, 1, mask)
     assert torch.equal(a, b) and torch.equal(la, lb)
+    # and without lse: the fast construction of the weights on both sides
+    qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, a, qs, ks, 1, 0, 2, D ** -0.5, 0, mask, two_waves=True)
+    qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, b, qs.repeat_interleave(8, dim=2).contiguous(),
+                                        ks.repeat_interleave(4, dim=2).contiguous(), 1, 0, 3, D ** -0.5, 0, mask)
+    assert torch.equal(a, b)
 
 
 def test_per_thread_argument_checks(dev):
