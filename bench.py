@@ -524,6 +524,21 @@ def main():
         t_path = event_time_ms(whole_path, reps, 2)
         path["whole_path_k_mean_prepare_attention_unpermute"] = {
             "ms": round(t_path, 4), "effective_tops": round(dense_ops / (t_path * 1e-3) / 1e12, 1)}
+        # the same sequence captured once as a HIP graph and replayed: what a serving loop pays per layer when the
+        # launches (six kernels and the allocations between them) come from one graph launch instead of from Python
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            whole_path()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            whole_path()
+        t_graph = event_time_ms(graph.replay, reps, 2)
+        path["whole_path_hip_graph_replay"] = {
+            "ms": round(t_graph, 4), "effective_tops": round(dense_ops / (t_graph * 1e-3) / 1e12, 1)}
+        del graph
 
     result = {
         "metric": METRIC_NAMES[args.workload],
