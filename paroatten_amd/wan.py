@@ -44,6 +44,13 @@ def permute_attn_out(attn_out, permute_plan, i_block, grid=(21, 45, 80), n_text=
 class PARO_WanAttnProcessor2_0(_ParoProcessorBase):
     def _tables(self, rotary_emb, device, head_dim):
         # (shared by all the processors of the model: the rotary tensor of a step is converted once)
+        if isinstance(rotary_emb, (tuple, list)):
+            # later diffusers versions hand over (cos, sin) as real tensors [1, N, 1, D] with the frequency of
+            # every channel pair repeated over the pair: already the kernel's form
+            cos_t, sin_t = rotary_emb
+            return SHARED_TABLES.get((cos_t, sin_t), device,
+                                     lambda: (cos_t.reshape(-1, head_dim).float().contiguous(),
+                                              sin_t.reshape(-1, head_dim).float().contiguous()))
         return SHARED_TABLES.get((rotary_emb,), device,
                                  lambda: rope.complex_to_real_tables(rotary_emb.reshape(-1, head_dim // 2)))
 

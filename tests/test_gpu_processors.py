@@ -217,6 +217,13 @@ def test_wan_processor_against_oracle(dev):
     assert cosine(out.cpu(), ref.cpu()) >= 0.999
     assert _rel_rms(out, ref) <= 0.05
 
+    # later diffusers versions pass (cos, sin) as real tensors [1, N, 1, D], every pair's frequency repeated over
+    # the pair: the same tables, hence the same bits
+    fr = freqs.reshape(N, D // 2)
+    pair = (fr.real.float().repeat_interleave(2, dim=1).view(1, N, 1, D).to(dev),
+            fr.imag.float().repeat_interleave(2, dim=1).view(1, N, 1, D).to(dev))
+    assert torch.equal(proc(attn, hidden, rotary_emb=pair), out)
+
     # cross-attention inputs (another key length) take the dense path
     ctx = torch.randn(B, 40, H * D, generator=g).to(dev, dtype)
     out_x = proc(attn, hidden, encoder_hidden_states=ctx)
