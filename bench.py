@@ -446,6 +446,13 @@ def main():
                 t_16 = event_time_ms(attn_pv16, max(10, reps // 4), 2)
                 dens[str(d)]["attn_kernel_ms_pv_f16"] = round(t_16, 4)
                 del v16
+                # scales of the per-thread granularity (qk_quant_gran 3) on the same inputs: the two-wave kernel in
+                # its plain launch form with two score-to-exponent maps per block
+                tq8, tqs, tk8, tks = Q.per_thread_int8(qp, kp, km)
+                t_pt = event_time_ms(lambda: attn_only(masks[d], L.PARO_ATTN_QK_PER_THREAD,
+                                                       operands=(tq8, tk8, av8_, tqs, tks)), reps, 2)
+                dens[str(d)]["attn_kernel_ms_per_thread_scales"] = round(t_pt, 4)
+                del tq8, tk8
     if not args.headline_only:
         # the same number of blocks per row as one contiguous run round the diagonal (not a benchmark
         # configuration: it shows what the mask FAMILY costs when a head's K8 + V8 exceed the L2)
