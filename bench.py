@@ -447,7 +447,7 @@ def main():
                 dens[str(d)]["attn_kernel_ms_pv_f16"] = round(t_16, 4)
                 del v16
                 # scales of the per-thread granularity (qk_quant_gran 3) on the same inputs: the two-wave kernel in
-                # its plain launch form with two score-to-exponent maps per block
+                # the launch form the library picks, with two score-to-exponent maps per block
                 tq8, tqs, tk8, tks = Q.per_thread_int8(qp, kp, km)
                 t_pt = event_time_ms(lambda: attn_only(masks[d], L.PARO_ATTN_QK_PER_THREAD,
                                                        operands=(tq8, tk8, av8_, tqs, tks)), reps, 2)

@@ -65,7 +65,7 @@ extern "C" {
                                  csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133, shapes :1034-1038): q_scale
                                  [B,H,nbq*2*8], scale g of a 32-row group for its rows r with r % 8 == g; k_scale
                                  [B,Hkv,nbk*4] (16-byte aligned), scale j of a 64-key block for its keys c with
-                                 (c % 8) / 2 == j.  Two-wave kernel, plain launch; with
+                                 (c % 8) / 2 == j.  Two-wave kernel; with
                                  neither PARO_ATTN_PV_F16 nor s_dump.  paro_quant_int8_per_thread makes such scales. */
 
 /* Version of this ABI (bumped when a signature changes or an export leaves the library; currently 2). */

@@ -15,7 +15,7 @@ Differences, all relaxations or added checks:
     accumulation, as the reference's kernel of this name computes it, instead of FP8 e4m3 P and V: true
     exponentials, V as given (smooth_v has nothing to act on); about half the speed;
   * `qk_quant_gran=3` (per thread: eight q scales per 32 rows, four k scales per 64 keys, indexed as
-    csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133) runs the two-wave kernel in its plain launch form;
+    csrc/qattn/qk_int_sv_f16_cuda_sm80.cu:112-116, 129-133) runs the two-wave kernel;
     quant.per_thread_int8 makes such scales (the reference has no quantiser for them);
   * keyword `pacing=True/False` picks the launch form of the attention kernel (see PARO_ATTN_PACED in
     include/paroatten.h; bit-identical results), None leaves it to the library;

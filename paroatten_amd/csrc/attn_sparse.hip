@@ -685,7 +685,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD) attn_sparse_ker
 // q-blocks of equal length, sorted by a pre-pass over the mask, changed nothing: a workgroup that waits leaves
 // the matrix pipe to its neighbours on the compute unit, so the waiting itself costs little.)
 constexpr int PACE_PAD = 32;   // counters 128 bytes apart: one per XCD
-template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT>
+template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT, bool PT = false>
 __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
     attn_sparse_paced_kernel(const AttnParams p, unsigned* __restrict__ counters, const int per, const int spin_limit,
                              const int slack) {
@@ -695,7 +695,7 @@ __global__ void __launch_bounds__(128, PARO_ATTN_WAVES_PER_SIMD)
   bool waiting = true;   // a workgroup that has once waited in vain goes on without waiting for the rest of the launch
   for (int base = first; base < last; base += G) {
     const int vid = base + slot;
-    if (vid < last) attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>(p, vid);
+    if (vid < last) attn_qblock<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT, PT>(p, vid);
     if (base + G >= last) break;
     // every workgroup of the XCD arrives once per generation, with or without a q-block of its own
     __syncthreads();   // also: both waves are done with this q-block's lists in LDS
@@ -769,8 +769,10 @@ static size_t attn_list_bytes(int nbk, int list_pad, bool per_thread) {
 template <int D, int OUT_DT, bool CAUSAL, bool DUMP, bool LSE, bool EXACT, bool PT = false>
 static int launch_attn(const AttnParams& p, hipStream_t st) {
   const size_t smem = AttnLds<D>::LIST_OFF + attn_list_bytes(p.nbk, AttnLds<D>::LIST_PAD, PT);
-  if (!DUMP && !PT && want_pacing(p, D)) {
-    auto kern = attn_sparse_paced_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT>;
+  // (per-thread scales make the list three times as long: where that costs a compute unit its fourth workgroup,
+  // Wan 720p, the paced form with half the waves measured slower than the plain launch, 21.8 against 17.3 ms)
+  if (!DUMP && want_pacing(p, D) && (!PT || smem <= 40 * 1024)) {
+    auto kern = attn_sparse_paced_kernel<D, OUT_DT, CAUSAL, DUMP, LSE, EXACT, PT>;
     if (smem > 48 * 1024)
       PARO_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
     PaceDevice pd;
@@ -806,7 +808,7 @@ static int launch_attn(const AttnParams& p, hipStream_t st) {
   return PARO_OK;
 }
 
-// per-thread scales (qk_quant_gran 3): the two-wave kernel, plain launch
+// per-thread scales (qk_quant_gran 3): the two-wave kernel
 template <int D, int OUT_DT>
 static int dispatch_attn_per_thread(const AttnParams& p, int is_causal, bool exact, hipStream_t st) {
   if (p.lse != nullptr)

@@ -104,6 +104,23 @@ def test_per_thread_with_group_constant_scales_is_the_per_warp_kernel(dev):
     assert torch.equal(a, b)
 
 
+def test_per_thread_paced_launch_is_bit_identical(dev):
+    """the paced launch form with per-thread scales (more q-blocks per XCD than resident workgroups, so the generation
+    counters are in use): the same bits as the plain launch"""
+    from paroatten_amd import _qattn_sm80 as qattn, quant as Q
+    B, H, N, D = 2, 12, 3104, 128
+    q, k, v = (t.to(dev) for t in _inputs(B, H, H, N, D, torch.bfloat16, seed=3))
+    nb = (N + 63) // 64
+    mask = synth.make_block_mask(H, nb, 0.4, seed=5).to(dev)
+    q8, qs, k8, ks = Q.per_thread_int8(q, k)
+    outs = []
+    for pacing in (False, True):
+        o = torch.empty_like(q)
+        qattn.qk_int8_sv_f16_accum_f16_attn(q8, k8, v, o, qs, ks, 1, 0, 3, D ** -0.5, 0, mask, pacing=pacing)
+        outs.append(o)
+    assert torch.equal(outs[0], outs[1]) and bool(torch.isfinite(outs[0].float()).all())
+
+
 def test_per_thread_argument_checks(dev):
     from paroatten_amd import _qattn_sm80 as qattn, quant as Q
     import paroatten_amd as P
