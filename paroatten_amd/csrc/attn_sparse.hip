@@ -330,9 +330,11 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     load_v(kb_1, 1);
   }
   // (PT: the lane's two k scales of the block, for its even and its odd pairs of keys)
-  constexpr int CO = PT ? 1 : 0;
+  // (everything the odd pairs need is declared for PT only in effect: without PT the names below are never read,
+  // so the per-warp kernels are the instruction streams they were)
   float c_cur = qsc * clist[PT ? 2 * lh : 0];
-  float cb_cur = qsc * clist[CO * (2 * lh + 1)];
+  float cb_cur = 0.f;
+  if constexpr (PT) cb_cur = qsc * clist[2 * lh + 1];
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   read_k_frags(0);
@@ -376,17 +378,20 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     }
     const int kidx_v = (int)klist[it + 4];
     const float c_next = qsc * clist[(it + 1) * CW + (PT ? 2 * lh : 0)];
-    const float cb_next = qsc * clist[(it + 1) * CW + CO * (2 * lh + 1)];
+    float cb_next = 0.f;
+    if constexpr (PT) cb_next = qsc * clist[(it + 1) * CW + 2 * lh + 1];
     // scale of this block and what follows from it and from the current maximum alone
     const float c = c_cur;
-    const float cb = PT ? cb_cur : c;
+    const float cb = cb_cur;
     const float nmc = -S_MAGIC_F * c;
     const float c8 = (8.0f * FAST_FIELD_SCALE) * c;
     float bias = fmaf(-S_MAGIC_F, c, m_off);      // exact path:  t  = S*c - m + OFFSET
-    float biasb = fmaf(-S_MAGIC_F, cb, m_off);
+    float biasb = 0.f;
+    if constexpr (PT) biasb = fmaf(-S_MAGIC_F, cb, m_off);
     float bias8 = fmaf(-S_MAGIC_F, c8, m_off8);   // fast path: field = (8*(t + 7) + shift + 0.5) * 256 / 32767
-    const float c8b = PT ? (8.0f * FAST_FIELD_SCALE) * cb : c8;
-    float bias8b = fmaf(-S_MAGIC_F, c8b, m_off8);
+    const float c8b = (8.0f * FAST_FIELD_SCALE) * cb;
+    float bias8b = 0.f;
+    if constexpr (PT) bias8b = fmaf(-S_MAGIC_F, c8b, m_off8);
 
     float s[2][16];
 #pragma unroll
@@ -455,9 +460,9 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       m_off = P_EXP_OFFSET - m_new;
       m_off8 = (8.0f * (P_EXP_OFFSET + 7.0f - m_new) + FAST_EXP_SHIFT + 0.5f) * FAST_FIELD_SCALE;
       bias = fmaf(-S_MAGIC_F, c, m_off);
-      biasb = fmaf(-S_MAGIC_F, cb, m_off);
+      if constexpr (PT) biasb = fmaf(-S_MAGIC_F, cb, m_off);
       bias8 = fmaf(-S_MAGIC_F, c8, m_off8);
-      bias8b = fmaf(-S_MAGIC_F, c8b, m_off8);
+      if constexpr (PT) bias8b = fmaf(-S_MAGIC_F, c8b, m_off8);
       if constexpr (LSE) d_exact *= alpha;
       d_acc[0] *= alpha;                                          // lanes 0..15: q-row lane
       d_acc[1] *= __shfl(alpha, (lane & 15) + 16, 64);            // and q-row lane+16
@@ -490,7 +495,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
       auto fast_words = [&]() {
         float u_cur[4], u_nxt[4];
 #pragma unroll
-        for (int q = 0; q < 4; q++) u_cur[q] = fma_clamp01(s[0][q], q < 2 ? c8 : c8b, q < 2 ? bias8 : bias8b);
+        for (int q = 0; q < 4; q++)
+          u_cur[q] = fma_clamp01(s[0][q], PT && q >= 2 ? c8b : c8, PT && q >= 2 ? bias8b : bias8);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int r = 0; r < 8; r++) {
@@ -499,13 +505,13 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
           const int rn = r + 1, mtn = rn >> 2, in0 = 4 * (rn & 3);
           if (rn < 8) {
             u_nxt[0] = fma_clamp01(s[mtn][in0 + 0], c8, bias8);
-            u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], c8b, bias8b);
+            u_nxt[2] = fma_clamp01(s[mtn][in0 + 2], PT ? c8b : c8, PT ? bias8b : bias8);
           }
           const int lo = cvt_pknorm_i16(u_cur[0], u_cur[2]);
           __builtin_amdgcn_sched_barrier(0);
           if (rn < 8) {
             u_nxt[1] = fma_clamp01(s[mtn][in0 + 1], c8, bias8);
-            u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], c8b, bias8b);
+            u_nxt[3] = fma_clamp01(s[mtn][in0 + 3], PT ? c8b : c8, PT ? bias8b : bias8);
           }
           const int hi = cvt_pknorm_i16(u_cur[1], u_cur[3]);
           __builtin_amdgcn_sched_barrier(0);
@@ -542,8 +548,8 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
         const int mt = r >> 2, i0 = 4 * (r & 3);
         const float p0 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 0], c, bias));
         const float p1 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 1], c, bias));
-        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], cb, biasb));
-        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], cb, biasb));
+        const float p2 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 2], PT ? cb : c, PT ? biasb : bias));
+        const float p3 = __builtin_amdgcn_exp2f(fmaf(s[mt][i0 + 3], PT ? cb : c, PT ? biasb : bias));
         if constexpr (LSE) rs += (p0 + p1) + (p2 + p3);
         int w;
         cvt_pk_fp8<false>(w, p0, p1);
@@ -594,7 +600,7 @@ __device__ __forceinline__ void attn_qblock(const AttnParams& p, const int vid) 
     __builtin_amdgcn_s_barrier();
     kb_c = kb_1; kb_1 = kb_2; kb_2 = kb_3; kb_3 = kb_4;
     c_cur = c_next;
-    cb_cur = cb_next;
+    if constexpr (PT) cb_cur = cb_next;
   };
 
   if constexpr (RING2) {
